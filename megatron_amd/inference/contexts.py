@@ -18,7 +18,8 @@ large (256 tokens) to keep block tables small and gathers coalesced.
 from __future__ import annotations
 
 import math
-from typing import List, Optional, Tuple
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
 
@@ -368,3 +369,138 @@ class DynamicInferenceContext:
                             slot_grid, "v")
         out = _masked_decode_attention(q[0], k_gath, v_gath, new_lens, scale)
         return out.unsqueeze(0)
+
+
+# ---------------------------------------------------------------------------
+# ragged batches over paged caches AND recurrent state slots
+# ---------------------------------------------------------------------------
+
+
+class StateSlotAllocator:
+    """Free-list of fixed-size recurrent-state slots, one per live request.
+
+    Recurrent mixers (gated linear recurrences, matrix memories), short
+    convolutions and the embedding's previous-token register keep O(1) state
+    per sequence; a slot is the row index of that state in every per-layer
+    state tensor.  Slots are reused: the context zeroes a slot on admission."""
+
+    def __init__(self, num_slots: int):
+        self.num_slots = num_slots
+        self._free = list(range(num_slots - 1, -1, -1))
+
+    @property
+    def num_free(self) -> int:
+        return len(self._free)
+
+    def allocate(self) -> int:
+        if not self._free:
+            raise RuntimeError("out of state slots")
+        return self._free.pop()
+
+    def free(self, slot: int):
+        self._free.append(slot)
+
+
+@dataclass
+class RaggedBatch:
+    """Device-side layout of one mixed step: R requests, each bringing a
+    contiguous run of new tokens (a prompt portion or one decoded token),
+    flattened to T tokens.  Every ragged kernel reads this one descriptor."""
+
+    num_requests: int
+    num_tokens: int
+    cu_tokens: torch.Tensor     # [R+1] int32: token range of request r in the flat batch
+    start_pos: torch.Tensor     # [R]   int32: tokens the request already holds
+    slots: torch.Tensor         # [R]   int32: recurrent-state slot
+    block_tables: torch.Tensor  # [R, max_blocks] int32 (padded with 0)
+    tok_req: torch.Tensor       # [T]   int32: request row of each token
+    tok_pos: torch.Tensor       # [T]   int32: position of each token in its sequence
+    tok_row: torch.Tensor       # [T]   int64: flat cache row (block * block_size + offset)
+    max_new: int                # longest run of new tokens
+    max_context: int            # longest context after this step
+    block_size: int
+    # host copies, for reference code and launch geometry
+    host_cu: List[int] = None
+    host_start: List[int] = None
+    host_slots: List[int] = None
+    host_tables: List[List[int]] = None
+
+
+class HybridInferenceContext:
+    """Cache and state manager for models that mix attention over a paged
+    cache with recurrent layers.
+
+    * ``cache_specs``: name -> row width.  One paged pool per name,
+      ``[num_blocks * block_size, width]`` in the compute dtype, addressed by the
+      request's block table (all pools share the table: one page id covers
+      the same token range in every pool).
+    * ``state_specs``: name -> (per-slot shape, dtype).  One tensor per name,
+      ``[num_slots, *shape]``; recurrent state is kept in 32-bit floats whatever
+      the compute dtype.
+
+    The engine owns which request holds which pages and slot; layers get the
+    pools / state tensors by name and a :class:`RaggedBatch`."""
+
+    def __init__(self, cache_specs: Dict[str, int], state_specs: Dict[str, Tuple[Sequence[int], torch.dtype]],
+                 num_blocks: int, block_size: int, num_slots: int,
+                 dtype=torch.bfloat16, device="cuda"):
+        self.block_size = block_size
+        self.num_blocks = num_blocks
+        self.device = torch.device(device)
+        self.compute_dtype = dtype
+        self.allocator = KVBlockAllocator(num_blocks, first_id=0)
+        self.slot_allocator = StateSlotAllocator(num_slots)
+        self.pools = {name: torch.zeros(num_blocks * block_size, width, dtype=dtype, device=device)
+                      for name, width in cache_specs.items()}
+        self.states = {name: torch.zeros(num_slots, *shape, dtype=sdt, device=device)
+                       for name, (shape, sdt) in state_specs.items()}
+        self.batch: Optional[RaggedBatch] = None
+
+    # -- slots ------------------------------------------------------------
+
+    def acquire_slot(self) -> int:
+        """A zeroed state slot (a reused slot forgets its previous owner)."""
+        slot = self.slot_allocator.allocate()
+        for t in self.states.values():
+            t[slot].zero_()
+        return slot
+
+    def release_slot(self, slot: int):
+        self.slot_allocator.free(slot)
+
+    # -- step layout --------------------------------------------------------
+
+    def begin_batch(self, counts: List[int], starts: List[int], slots: List[int],
+                    tables: List[List[int]]) -> RaggedBatch:
+        """counts[r] new tokens for a request that already holds starts[r]."""
+        R = len(counts)
+        bs = self.block_size
+        cu = [0]
+        for c in counts:
+            cu.append(cu[-1] + c)
+        T = cu[-1]
+        maxb = max(1, max(len(t) for t in tables))
+        bt = torch.zeros(R, maxb, dtype=torch.int32)
+        for r, t in enumerate(tables):
+            need = (starts[r] + counts[r] + bs - 1) // bs
+            assert len(t) >= need, "request holds too few pages for this step"
+            bt[r, : len(t)] = torch.as_tensor(t, dtype=torch.int32)
+        tok_req = torch.repeat_interleave(torch.arange(R, dtype=torch.int32),
+                                          torch.as_tensor(counts, dtype=torch.long))
+        cu_t = torch.as_tensor(cu, dtype=torch.int32)
+        start_t = torch.as_tensor(starts, dtype=torch.int32)
+        tok_pos = (torch.arange(T, dtype=torch.int32) - cu_t[:-1][tok_req.long()]
+                   + start_t[tok_req.long()])
+        blk = bt[tok_req.long(), (tok_pos // bs).long()].long()
+        tok_row = blk * bs + (tok_pos % bs).long()
+        dev = self.device
+        self.batch = RaggedBatch(
+            num_requests=R, num_tokens=T,
+            cu_tokens=cu_t.to(dev), start_pos=start_t.to(dev),
+            slots=torch.as_tensor(slots, dtype=torch.int32).to(dev),
+            block_tables=bt.to(dev), tok_req=tok_req.to(dev), tok_pos=tok_pos.to(dev),
+            tok_row=tok_row.to(dev), max_new=max(counts),
+            max_context=max(s + c for s, c in zip(starts, counts)), block_size=bs,
+            host_cu=cu, host_start=list(starts), host_slots=list(slots),
+            host_tables=[list(t) for t in tables])
+        return self.batch

@@ -19,7 +19,11 @@ from typing import Dict, List, Optional, Sequence
 import torch
 import torch.distributed as dist
 
-from megatron_amd.inference.contexts import DynamicInferenceContext, StaticInferenceContext
+from megatron_amd.inference.contexts import (
+    DynamicInferenceContext,
+    HybridInferenceContext,
+    StaticInferenceContext,
+)
 from megatron_amd.inference.sampling import SamplingParams, log_prob_of, sample
 from megatron_amd.parallel import grid as G
 from megatron_amd.parallel.mappings import gather_from_tensor_model_parallel_region
@@ -368,6 +372,7 @@ class _Request:
     cached: int = 0          # prompt tokens already in the KV cache
     next_input: Optional[int] = None  # token to feed at the next decode step
     gen: Optional[torch.Generator] = None
+    slot: Optional[int] = None  # recurrent-state slot (ragged-batch models)
 
 
 class DynamicInferenceEngine:
@@ -383,30 +388,42 @@ class DynamicInferenceEngine:
         device = device or next(model.parameters()).device
         self.device = device
         self.eod = tokenizer.eod if tokenizer is not None else cfg.vocab_size - 1
+        self.max_batch = max_batch
+        self.max_prefill_tokens = max_prefill_tokens
+        assert scheduling_policy in ("fcfs", "priority", "sjf")
+        self.scheduling_policy = scheduling_policy
+        self._graphs = None
+        self._ids = itertools.count()
+        self.waiting: List[_Request] = []
+        self.active: List[_Request] = []
+        self.finished: Dict[int, GenerationResult] = {}
+        self.preempted: List[tuple] = []
+        # models with recurrent layers / their own cache rows describe what
+        # they need (inference_spec) and run ragged mixed batches: portions of
+        # prompts beside single decoded tokens in ONE forward per step
+        self.ragged = bool(getattr(model, "ragged_batch", False))
+        if self.ragged:
+            spec = model.inference_spec()
+            self.context = HybridInferenceContext(
+                spec.caches, spec.states, num_blocks=num_blocks, block_size=block_size,
+                num_slots=max_batch, dtype=cfg.params_dtype, device=device)
+            self.prefix_caching = False   # recurrent state cannot be rebuilt from shared pages
+            self.offloader = None
+            return
         tp = G.get_tensor_model_parallel_world_size()
         self.context = DynamicInferenceContext(
             cfg.num_layers,
             (cfg.num_query_groups or cfg.num_attention_heads) // tp,
             cfg.kv_channels, num_blocks=num_blocks, block_size=block_size,
             dtype=cfg.params_dtype, device=device, kv_cache_dtype=kv_cache_dtype)
-        self.max_batch = max_batch
-        self.max_prefill_tokens = max_prefill_tokens
-        assert scheduling_policy in ("fcfs", "priority", "sjf")
-        self.scheduling_policy = scheduling_policy
-        self._graphs = None
         pp = G.get_grid().pp if G.grid_initialized() else 1
         if (use_hip_graphs and torch.cuda.is_available() and device.type == "cuda"
                 and tp == 1 and pp == 1):
             self._graphs = _DecodeGraphRunner(self.model, self.context, device)
-        self._ids = itertools.count()
-        self.waiting: List[_Request] = []
-        self.active: List[_Request] = []
-        self.finished: Dict[int, GenerationResult] = {}
         # host-offload preemption (LIFO preempt, FIFO restore)
         from megatron_amd.inference.offload import KVHostOffloader
 
         self.offloader = KVHostOffloader(self.context)
-        self.preempted: List[tuple] = []  # (req, handle)
         self.prefix_caching = enable_prefix_caching
         if enable_prefix_caching:
             from megatron_amd.inference.contexts import PrefixCachingAllocator
@@ -448,8 +465,7 @@ class DynamicInferenceEngine:
             for req in q:
                 if req.rid == rid:
                     q.remove(req)
-                    self.context.allocator.free(req.block_table)
-                    req.block_table = []
+                    self._release(req)
                     req.result.finished = True
                     req.result.aborted = True
                     self.finished[rid] = req.result
@@ -572,9 +588,16 @@ class DynamicInferenceEngine:
         text = self.tokenizer.detokenize(req.result.output_tokens)
         return any(text.endswith(ss) for ss in req.params.stop_strings)
 
-    def _finish(self, req: _Request):
+    def _release(self, req: _Request):
+        """Give a request's pages (and state slot) back for reuse."""
         self.context.allocator.free(req.block_table)
         req.block_table = []
+        if req.slot is not None:
+            self.context.release_slot(req.slot)
+            req.slot = None
+
+    def _finish(self, req: _Request):
+        self._release(req)
         req.result.finished = True
         if self.tokenizer is not None:
             req.result.text = self.tokenizer.detokenize(req.result.output_tokens)
@@ -597,7 +620,10 @@ class DynamicInferenceEngine:
     @torch.no_grad()
     def step(self) -> None:
         """One engine step: chunked prefill of the next waiting request, or one
-        batched decode step over all active requests."""
+        batched decode step over all active requests.  Ragged-batch models run
+        both kinds of work in one forward (see _step_ragged)."""
+        if self.ragged:
+            return self._step_ragged()
         self._restore_preempted()
         if self.waiting and len(self.active) < self.max_batch:
             req = self._next_waiting()
@@ -679,6 +705,117 @@ class DynamicInferenceEngine:
             else:
                 tok = self._sample_row(logits[i], req)
             req.result.output_tokens.append(tok)
+            if req.params.stop_on_eod and tok == self.eod:
+                req.result.output_tokens.pop()
+                self._finish(req)
+            elif self._hit_stop_string(req):
+                self._finish(req)
+            elif len(req.result.output_tokens) >= req.params.max_tokens:
+                self._finish(req)
+            else:
+                req.next_input = tok
+                still.append(req)
+        self.active = still
+
+    # -- ragged mixed batches (models with ragged_batch = True) -----------------
+
+    def open_request(self, params: SamplingParams = SamplingParams()) -> _Request:
+        """Admit a request whose tokens the caller feeds itself through
+        forward_batch (scoring / replay of given token streams): takes a state
+        slot now, pages as tokens arrive.  close_request gives both back."""
+        assert self.ragged, "externally fed requests need a ragged-batch model"
+        rid = next(self._ids)
+        req = _Request(rid, [], params, GenerationResult(rid, []))
+        req.slot = self.context.acquire_slot()
+        return req
+
+    def close_request(self, req: _Request):
+        self._release(req)
+
+    @torch.no_grad()
+    def forward_batch(self, feeds, want=None) -> Optional[torch.Tensor]:
+        """The step function of ragged-batch models: run every (request, new
+        tokens) pair of ``feeds`` in ONE forward from the caches and states
+        earlier steps left, and advance them.  ``want[i]`` lists the places
+        among feeds[i]'s tokens whose logits are returned ([n, vocab] fp32, in
+        feed order); default: each feed's last token."""
+        ctx = self.context
+        counts, starts, slots, tables, flat, rows = [], [], [], [], [], []
+        base = 0
+        for i, (req, toks) in enumerate(feeds):
+            n = len(toks)
+            assert n > 0, "a feed brings at least one token"
+            if req.cached + n > self.model.config.max_position_embeddings:
+                raise RuntimeError("request exceeds the model's position range")
+            if not self._ensure_blocks(req, req.cached + n):
+                raise RuntimeError("cache pool exhausted")
+            counts.append(n)
+            starts.append(req.cached)
+            slots.append(req.slot)
+            tables.append(req.block_table)
+            flat.extend(toks)
+            rows.extend(base + w for w in (want[i] if want is not None else [n - 1]))
+            base += n
+        ctx.begin_batch(counts, starts, slots, tables)
+        tokens = torch.as_tensor(flat, dtype=torch.long).to(self.device)
+        for (req, toks), n in zip(feeds, counts):
+            req.cached += n
+        if not rows:
+            # nothing asked for: still run the step (it fills caches and states)
+            self.model(tokens, inference_context=ctx,
+                       want=torch.zeros(1, dtype=torch.long, device=self.device))
+            return None
+        return self.model(tokens, inference_context=ctx,
+                          want=torch.as_tensor(rows, dtype=torch.long).to(self.device))
+
+    def _step_ragged(self) -> None:
+        """Continuous batching with mixed steps: every active request decodes
+        one token and waiting prompts are fed in portions, all in one forward,
+        under a per-step token budget (max_prefill_tokens) and the slot count
+        (max_batch).  A prompt whose next portion finds no free pages waits."""
+        ctx = self.context
+        feeds, kinds = [], []
+        budget = self.max_prefill_tokens
+        for req in self.active:
+            if not self._ensure_blocks(req, req.cached + 1):   # decodes reserve before prompts
+                raise RuntimeError("cache pool exhausted by running requests")
+            feeds.append((req, [req.next_input]))
+            kinds.append("decode")
+            budget -= 1
+        order = list(self.waiting)
+        if self.scheduling_policy != "fcfs":
+            order.sort(key=lambda r: (getattr(r, "priority", 0),
+                                      len(r.prompt) if self.scheduling_policy == "sjf" else 0, r.rid))
+        for req in order:
+            if budget <= 0:
+                break
+            if req.slot is None:
+                if ctx.slot_allocator.num_free == 0:
+                    continue
+                req.slot = ctx.acquire_slot()
+            n = min(budget, len(req.prompt) - req.cached)
+            bs = ctx.block_size
+            have = len(req.block_table) * bs - req.cached
+            n = min(n, have + ctx.allocator.num_free * bs)
+            if n <= 0:
+                continue
+            self._ensure_blocks(req, req.cached + n)   # reserve now: later feeds see the rest
+            feeds.append((req, req.prompt[req.cached:req.cached + n]))
+            kinds.append("prefill")
+            budget -= n
+        if not feeds:
+            if self.waiting:
+                raise RuntimeError("cache pool too small for a single prompt portion")
+            return
+        logits = self.forward_batch(feeds)          # last place of every feed
+        still = []
+        for i, ((req, toks), kind) in enumerate(zip(feeds, kinds)):
+            if kind == "prefill" and req.cached < len(req.prompt):
+                continue                            # prompt not finished: logits unused
+            tok = self._sample_row(logits[i], req)
+            req.result.output_tokens.append(tok)
+            if kind == "prefill":
+                self.waiting.remove(req)
             if req.params.stop_on_eod and tok == self.eod:
                 req.result.output_tokens.pop()
                 self._finish(req)

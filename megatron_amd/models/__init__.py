@@ -19,4 +19,8 @@ def __getattr__(name):  # lazy: bert/t5/llava/audio pull heavier deps
         from megatron_amd.models.audio import AudioLanguageModel
 
         return AudioLanguageModel
+    if name in ("BezutarModel", "BezutarConfig"):
+        from megatron_amd.models import bezutar
+
+        return getattr(bezutar, name)
     raise AttributeError(name)

@@ -1,0 +1,232 @@
+"""Torch implementations of the ragged-batch sequence ops (CPU path).
+
+Every op works on a flat batch of T tokens described by a
+``RaggedBatch`` (megatron_amd/inference/contexts.py): request r brings tokens
+``cu_tokens[r]:cu_tokens[r+1]`` at positions ``start_pos[r]...``; per-sequence
+state lives in ``[num_slots, ...]`` tensors indexed by ``slots[r]`` and is
+updated in place; paged caches are ``[rows, width]`` pools addressed through the
+block tables.  The HIP kernels in csrc/ragged implement the same interfaces.
+
+Precision rules (same as the kernels): norms, recurrences, gates, angles,
+scores and softmax weights are computed in 32-bit whatever the tensors'
+storage dtype; outputs are rounded once, on store.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn.functional as F
+
+
+def _spans(batch):
+    for r in range(batch.num_requests):
+        yield r, batch.host_cu[r], batch.host_cu[r + 1], batch.host_start[r], batch.host_slots[r]
+
+
+def embed_tokens(tokens, batch, embed, bigram, pos, prev_state, mul_prev, mul_cur, buckets):
+    """x[t] = embed[tok] (+ bigram[hash(prev, tok)]) (+ pos[p]) in fp32.
+
+    The hashed-bigram row is ``(prev * mul_prev + tok * mul_cur) % buckets``; a
+    sequence's first token uses the extra row ``buckets``.  ``prev_state[slot]``
+    carries the last token across steps."""
+    x = embed[tokens].float()
+    if bigram is not None:
+        prev = torch.roll(tokens, 1)
+        first_idx = batch.cu_tokens[:-1].long()
+        prev[first_idx] = prev_state[batch.slots.long()].to(prev.dtype)
+        row = (prev * mul_prev + tokens * mul_cur) % buckets
+        row = torch.where(batch.tok_pos == 0, torch.full_like(row, buckets), row)
+        x = x + bigram[row].float()
+        last_idx = batch.cu_tokens[1:].long() - 1
+        prev_state[batch.slots.long()] = tokens[last_idx].to(prev_state.dtype)
+    if pos is not None:
+        x = x + pos[batch.tok_pos.long()].float()
+    return x
+
+
+def hc_mix_norm(streams, y, mix, out_w, in_w, norm_w, eps):
+    """Hyper-connection stream update fused with the next read and its norm.
+
+    streams [T, S, W] fp32 (updated in place when ``y`` is given):
+        x_t <- sum_s mix[s, t] x_s + out_w[t] * y
+    then, when ``in_w`` is given, u = sum_s in_w[s] x_s and the result is
+    ``u / sqrt(mean(u^2) + eps) * (1 + norm_w)`` in fp32 ([T, W])."""
+    if y is not None:
+        new = torch.einsum("st,nsw->ntw", mix.float(), streams) + out_w.float()[None, :, None] * y.float()[:, None, :]
+        streams.copy_(new)
+    if in_w is None:
+        return None
+    u = torch.einsum("s,nsw->nw", in_w.float(), streams)
+    u = u * torch.rsqrt((u * u).mean(-1, keepdim=True) + eps)
+    return u * (1.0 + norm_w.float())
+
+
+def canon_conv(h, weight, state, batch, out_dtype):
+    """h + causal depthwise conv over time of h, per request, with the last
+    ``taps - 1`` inputs of earlier steps read from (and left in) ``state``
+    [slots, taps-1, W].  weight [W, taps]: out_t = h_t + sum_j w[:, j] h_{t-taps+1+j}."""
+    taps = weight.shape[1]
+    out = torch.empty(h.shape, dtype=out_dtype, device=h.device)
+    wf = weight.float()
+    for r, a, b, start, slot in _spans(batch):
+        hist = torch.cat([state[slot], h[a:b].float()], dim=0)  # [taps-1 + n, W]
+        n = b - a
+        acc = h[a:b].float().clone()
+        for j in range(taps):
+            acc += wf[:, j] * hist[j : j + n]
+        out[a:b] = acc.to(out_dtype)
+        state[slot] = hist[n:]
+    return out
+
+
+def mingru_scan(zxg, bias_z, bias_x, state, batch, out_dtype):
+    """minGRU over a ragged batch.  zxg [T, 3C]: pre-activations of the update
+    gate, the candidate and the output gate.  z = sigmoid(. + bz); u = . + bx;
+    cand = u + 1/2 (u >= 0) | sigmoid(u); S <- (1 - z) S + z cand; out = S * silu(g).
+    state [slots, C] fp32."""
+    C = zxg.shape[1] // 3
+    z = torch.sigmoid(zxg[:, :C].float() + bias_z.float())
+    u = zxg[:, C : 2 * C].float() + bias_x.float()
+    g = zxg[:, 2 * C :].float()
+    cand = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
+    out = torch.empty(zxg.shape[0], C, dtype=torch.float32, device=zxg.device)
+    for r, a, b, start, slot in _spans(batch):
+        S = state[slot].clone()
+        for t in range(a, b):
+            S = (1 - z[t]) * S + z[t] * cand[t]
+            out[t] = S
+        state[slot] = S
+    return (out * F.silu(g)).to(out_dtype)
+
+
+def mlstm_scan(qkvg, gates, bias_i, bias_f, norm_w, heads, dim, vdim, cap, eps,
+               state_S, state_n, state_m, batch, out_dtype):
+    """Stabilised matrix-memory recurrence (mLSTM) over a ragged batch.
+
+    qkvg [T, H*dim | H*dim | H*vdim | H*vdim] (q unscaled, k, v, output-gate
+    pre-activation); gates [T, 2H] fp32 pre-activations of the input and forget
+    gates.  Log gates are soft-capped: i = cap tanh((. + bi)/cap),
+    f = logsigmoid(cap tanh((. + bf)/cap)).  With running maximum m (0 at start):
+        m' = max(f + m, i); S' = e^{f+m-m'} S + e^{i-m'} k v^T; n' likewise with k
+        o = S'^T q / (max(|n'.q|, e^{-m'}) + 1e-6),  q scaled by dim^-1/2.
+    Each head's o is RMS-normalised, scaled by norm_w and gated by sigmoid(g).
+    States: S [slots, H, dim, vdim], n [slots, H, dim], m [slots, H], fp32."""
+    T = qkvg.shape[0]
+    H, D, V = heads, dim, vdim
+    q, k, v, g = torch.split(qkvg.float(), [H * D, H * D, H * V, H * V], dim=1)
+    q = q.view(T, H, D) * (D ** -0.5)
+    k = k.view(T, H, D)
+    v = v.view(T, H, V)
+    ig = cap * torch.tanh((gates[:, :H].float() + bias_i.float()) / cap)
+    fg = F.logsigmoid(cap * torch.tanh((gates[:, H:].float() + bias_f.float()) / cap))
+    o = torch.empty(T, H, V, dtype=torch.float32, device=qkvg.device)
+    for r, a, b, start, slot in _spans(batch):
+        S, n, m = state_S[slot].clone(), state_n[slot].clone(), state_m[slot].clone()
+        for t in range(a, b):
+            m_new = torch.maximum(fg[t] + m, ig[t])
+            da = torch.exp(fg[t] + m - m_new)
+            db = torch.exp(ig[t] - m_new)
+            S = da[:, None, None] * S + db[:, None, None] * (k[t][:, :, None] * v[t][:, None, :])
+            n = da[:, None] * n + db[:, None] * k[t]
+            m = m_new
+            num = torch.einsum("hdv,hd->hv", S, q[t])
+            den = torch.maximum((n * q[t]).sum(-1).abs(), torch.exp(-m)) + 1e-6
+            o[t] = num / den[:, None]
+        state_S[slot], state_n[slot], state_m[slot] = S, n, m
+    o = o * torch.rsqrt((o * o).mean(-1, keepdim=True) + eps)
+    o = o.reshape(T, H * V) * norm_w.float() * torch.sigmoid(g)
+    return o.to(out_dtype)
+
+
+def rope_table(max_pos, dims, base, scaling=None, device=None):
+    """cos/sin tables [max_pos, dims/2] fp32 for rotate-half RoPE with optional
+    YaRN frequency interpolation.  scaling: dict(factor, original, fast, slow).
+    Frequencies are blended between f_i and f_i / factor by a linear ramp over
+    the pair index between the 'fast' and 'slow' rotation counts; cos and sin
+    carry the YaRN magnitude factor 0.1 ln(factor) + 1."""
+    half = dims // 2
+    f = torch.tensor([base ** (-2.0 * i / dims) for i in range(half)], dtype=torch.float64)
+    mag = 1.0
+    if scaling:
+        def pair_of(turns):
+            return dims * math.log(scaling["original"] / (2 * math.pi * turns)) / (2 * math.log(base))
+        lo = max(math.floor(pair_of(scaling["fast"])), 0)
+        hi = min(math.ceil(pair_of(scaling["slow"])), dims - 1)
+        ramp = ((torch.arange(half, dtype=torch.float64) - lo) / max(hi - lo, 0.001)).clamp(0, 1)
+        f = f / scaling["factor"] * ramp + f * (1 - ramp)
+        mag = 0.1 * math.log(scaling["factor"]) + 1.0
+    ang = torch.arange(max_pos, dtype=torch.float32)[:, None] * f.to(torch.float32)[None, :]
+    return (torch.cos(ang) * mag).to(device), (torch.sin(ang) * mag).to(device)
+
+
+def _rotate(x, cos, sin, dims):
+    half = dims // 2
+    u, v = x[..., :half], x[..., half:dims]
+    return torch.cat([u * cos - v * sin, v * cos + u * sin, x[..., dims:]], dim=-1)
+
+
+def latent_kv_store(dkv, norm_w, eps, cos, sin, rot_dims, rank, pool, batch):
+    """Write each token's cache row: [RMS-normed latent * norm_w | rotated
+    shared key part].  dkv [T, rank + rot_dim]; pool [rows, rank + rot_dim]."""
+    c = dkv[:, :rank].float()
+    c = c * torch.rsqrt((c * c).mean(-1, keepdim=True) + eps) * norm_w.float()
+    p = batch.tok_pos.long()
+    kr = _rotate(dkv[:, rank:].float(), cos[p], sin[p], rot_dims)
+    pool[batch.tok_row] = torch.cat([c, kr], dim=-1).to(pool.dtype)
+
+
+def latent_q_prepare(dq, norm_w, eps, out_dtype):
+    """RMS norm with a plain weight over the query latent."""
+    c = dq.float()
+    return (c * torch.rsqrt((c * c).mean(-1, keepdim=True) + eps) * norm_w.float()).to(out_dtype)
+
+
+def rope_heads(x, cos, sin, rot_dims, batch):
+    """Rotate the first rot_dims dims of every head.  x [T, H, d]."""
+    p = batch.tok_pos.long()
+    return _rotate(x.float(), cos[p][:, None, :], sin[p][:, None, :], rot_dims).to(x.dtype)
+
+
+def latent_sink_attention(q, pool, rank, sink, scale, batch):
+    """Causal attention of absorbed queries over the paged latent cache.
+
+    q [T, H, rank + rot] scores every cached row [latent | rotated key] of its
+    own request up to its position; values are the rows' first ``rank`` entries
+    (the value up-projection is applied by the caller).  The softmax
+    denominator also holds exp(sink[h]): a per-head logit with no key or value."""
+    T, H, Dk = q.shape
+    out = torch.empty(T, H, rank, dtype=torch.float32, device=q.device)
+    bs = batch.block_size
+    for r, a, b, start, slot in _spans(batch):
+        L = start + (b - a)
+        table = torch.as_tensor(batch.host_tables[r], dtype=torch.long, device=q.device)
+        rows = (table[:, None] * bs + torch.arange(bs, device=q.device)[None, :]).reshape(-1)[:L]
+        kv = pool[rows].float()                               # [L, Dk]
+        s = torch.einsum("thd,ld->thl", q[a:b].float(), kv) * scale
+        qpos = torch.arange(start, L, device=q.device)
+        mask = torch.arange(L, device=q.device)[None, :] > qpos[:, None]
+        s = s.masked_fill(mask[:, None, :], float("-inf"))
+        s = torch.cat([s, sink.float().view(1, H, 1).expand(b - a, H, 1)], dim=-1)
+        p = torch.softmax(s, dim=-1)[..., :L]
+        out[a:b] = torch.einsum("thl,lr->thr", p, kv[:, :rank])
+    return out.to(q.dtype)
+
+
+def xielu(z, act, out_dtype):
+    """xIELU with raw parameters act = (p, q): for z > 0, softplus(p) z^2 + z/2;
+    else (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2."""
+    zf = z.float()
+    ap = F.softplus(act[0].float())
+    aq = 0.5 + F.softplus(act[1].float())
+    pos = ap * zf * zf + 0.5 * zf
+    neg = aq * (torch.expm1(torch.clamp(zf, max=0.0)) - zf) + 0.5 * zf
+    return torch.where(zf > 0, pos, neg).to(out_dtype)
+
+
+def gate_heads(x, gate_pre, heads):
+    """x [T, H*d] times sigmoid(gate_pre [T, H]) per head."""
+    T = x.shape[0]
+    g = torch.sigmoid(gate_pre.float())
+    return (x.float().view(T, heads, -1) * g[:, :, None]).reshape(T, -1).to(x.dtype)

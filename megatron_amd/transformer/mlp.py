@@ -54,3 +54,23 @@ class MLP(nn.Module):
             h = self._act(h)
         out, _ = self.linear_fc2(h)
         return out
+
+
+class XieluMLP(nn.Module):
+    """Dense two-matrix feed-forward with the xIELU activation
+    (ops.ragged.xielu): for z > 0, softplus(p) z^2 + z/2; otherwise
+    (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2, with two learned raw scalars
+    ``act = (p, q)``.  Plain replicated weights (serving path)."""
+
+    def __init__(self, hidden: int, ffn: int, dtype=torch.bfloat16):
+        super().__init__()
+        self.w_up = nn.Parameter(torch.zeros(ffn, hidden, dtype=dtype))
+        self.w_down = nn.Parameter(torch.zeros(hidden, ffn, dtype=dtype))
+        self.act = nn.Parameter(torch.zeros(2, dtype=torch.float32))
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        import torch.nn.functional as F
+
+        from megatron_amd.ops import ragged as R
+
+        return F.linear(R.xielu(F.linear(h, self.w_up), self.act, h.dtype), self.w_down)
