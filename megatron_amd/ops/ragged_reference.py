@@ -226,7 +226,7 @@ def xielu(z, act, out_dtype):
 
 
 def gate_heads(x, gate_pre, heads):
-    """x [T, H*d] times sigmoid(gate_pre [T, H]) per head."""
+    """x [T, H, d] (any strides) times sigmoid(gate_pre [T, H]) per head -> [T, H*d]."""
     T = x.shape[0]
     g = torch.sigmoid(gate_pre.float())
-    return (x.float().view(T, heads, -1) * g[:, :, None]).reshape(T, -1).to(x.dtype)
+    return (x.float() * g[:, :, None]).reshape(T, -1).to(x.dtype)

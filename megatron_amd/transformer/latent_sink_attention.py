@@ -73,6 +73,6 @@ class LatentSinkAttention(nn.Module):
         q_abs = torch.bmm(q[..., :D].transpose(0, 1), self.w_uk).transpose(0, 1)  # [T, H, r]
         lat_q = R.assemble_latent_q(q_abs, q[..., D:], self.cos, self.sin, self.rot_dims, batch)
         c_hat = R.latent_sink_attention(lat_q, pool, r, self.sink, self.scale, batch)  # [T, H, r]
-        o = torch.bmm(c_hat.transpose(0, 1), self.w_uv.transpose(1, 2)).transpose(0, 1)  # [T, H, vd]
-        o = R.gate_heads(o.reshape(T, H * self.vdim), a[:, a.shape[1] - H :], H)
+        o = torch.bmm(c_hat.transpose(0, 1), self.w_uv.transpose(1, 2)).transpose(0, 1)  # [T, H, vd] view
+        o = R.gate_heads(o, a[:, a.shape[1] - H :], H)                                   # [T, H * vd]
         return F.linear(o, self.w_out)

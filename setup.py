@@ -28,24 +28,48 @@ SRC = [
     "megatron_amd/ops/csrc/symm_allreduce.hip",
 ]
 
-setup(
-    name="megatron_amd_hip_ops",
-    ext_modules=[
+# hipcc must not form packed-fp32 VALU ops on this hardware pool
+HIPCC_FLAGS = ["-O3", "-std=c++17", "--offload-arch=gfx950",
+               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+RAGGED_SRC = [
+    "megatron_amd/ops/csrc/ragged/bindings.cpp",
+    "megatron_amd/ops/csrc/ragged/streams.hip",
+    "megatron_amd/ops/csrc/ragged/recurrent.hip",
+    "megatron_amd/ops/csrc/ragged/latent_attention.hip",
+]
+
+# MEGATRON_AMD_ONLY_EXT=ragged builds just the serving kernels of the
+# ragged-batch models (what a fresh checkout compiles on first use)
+ONLY = os.environ.get("MEGATRON_AMD_ONLY_EXT", "")
+
+EXTS = {
+    "hip": lambda:
         CUDAExtension(
             name="megatron_amd.ops._hip_ops",
             sources=SRC,
             extra_compile_args={
                 "cxx": ["-O3", "-std=c++17"],
-                "nvcc": ["-O3", "-std=c++17", "--offload-arch=gfx950"]
-                + os.environ.get("MEGATRON_AMD_HIPCC_EXTRA", "").split(),
+                "nvcc": HIPCC_FLAGS + os.environ.get("MEGATRON_AMD_HIPCC_EXTRA", "").split(),
             },
             libraries=["rocblas", "hipblaslt"],
         ),
+    "ragged": lambda:
+        CUDAExtension(
+            name="megatron_amd.ops._ragged_ops",
+            sources=RAGGED_SRC,
+            extra_compile_args={"cxx": ["-O3", "-std=c++17"], "nvcc": HIPCC_FLAGS},
+        ),
+    "data": lambda:
         CppExtension(
             name="megatron_amd.datasets._data_helpers",
             sources=["megatron_amd/datasets/csrc/data_helpers.cpp"],
             extra_compile_args={"cxx": ["-O3", "-std=c++17"]},
         ),
-    ],
+}
+
+setup(
+    name="megatron_amd_hip_ops",
+    ext_modules=[make() for key, make in EXTS.items() if not ONLY or key in ONLY.split(",")],
     cmdclass={"build_ext": BuildExtension.with_options(use_ninja=True)},
 )
