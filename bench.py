@@ -82,6 +82,17 @@ def parse_args():
                    help="run hipBLASLt TunableOp algo search and save profiles/tunableop_gfx950.csv")
     p.add_argument("--no-tunableop", action="store_true",
                    help="skip loading the committed TunableOp GEMM selections")
+    # serving comparison (does not touch the default training workload)
+    p.add_argument("--serve", action="store_true",
+                   help="instead of the training step: prefill/decode throughput of the ragged-batch "
+                        "Bezutar design beside GPT with multi-latent attention at equal sizes")
+    p.add_argument("--serve-sizes", default="1b,7b-layers")
+    p.add_argument("--serve-patterns", default="AMGA,A",
+                   help="layer patterns of the new design: A latent attention, M mLSTM, G minGRU")
+    p.add_argument("--serve-batch", type=int, default=4)
+    p.add_argument("--serve-isl", type=int, default=2048)
+    p.add_argument("--serve-osl", type=int, default=64)
+    p.add_argument("--serve-skip-baseline", action="store_true")
     return p.parse_args()
 
 
@@ -119,6 +130,10 @@ def setup_tunableop(args, rank):
 
 def main():
     args = parse_args()
+    if args.serve:
+        from megatron_amd.inference.bench_serving import main as serve_main
+
+        return serve_main(args)
     world = int(os.environ.get("WORLD_SIZE", "1"))
     rank = int(os.environ.get("RANK", "0"))
     use_dist = world > 1 or "RANK" in os.environ

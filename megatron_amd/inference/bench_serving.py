@@ -1,0 +1,172 @@
+"""Serving throughput of ragged-batch models beside the closest dense model.
+
+For each size: random-init weights, bf16, synthetic prompts.  Prefill =
+``batch`` prompts of ``isl`` tokens run to their last token; decode = ``osl``
+steps of one token per request.  The new design runs through
+DynamicInferenceEngine.forward_batch (one mixed forward per step); the
+comparison model is GPTModel with multi-latent attention at the same width,
+depth, heads and ranks through the same engine class (its paged-latent path:
+one prompt per prefill step, batched decode steps).  One JSON line per
+(size, model), tokens/s for both phases.
+"""
+
+from __future__ import annotations
+
+import json
+import time
+
+import torch
+
+SIZES = {
+    # width, layers, heads, qk dim (unrotated), rot, vdim, kv_rank, q_rank, ff, mlstm heads/dim/vdim, mingru width
+    "1b": dict(width=2048, layers=8, heads=16, dim=64, rot=32, vdim=64, kv_rank=256, q_rank=768, ff=5632,
+               m_heads=4, m_dim=128, m_vdim=256, gru=4096, vocab=32000),
+    "7b-layers": dict(width=4096, layers=4, heads=32, dim=128, rot=64, vdim=128, kv_rank=512, q_rank=1536,
+                      ff=11008, m_heads=8, m_dim=256, m_vdim=512, gru=8192, vocab=32000),
+}
+
+
+def bezutar_config(s, pattern, max_pos):
+    att = dict(type="latent_attention",
+               mixer=dict(heads=s["heads"], dim=s["dim"], rot_dim=s["rot"], vdim=s["vdim"], kv_rank=s["kv_rank"],
+                          q_rank=s["q_rank"], scale=(s["dim"] + s["rot"]) ** -0.5,
+                          rot=dict(base=10000.0, dims=s["rot"],
+                                   scaling=dict(factor=4.0, original=max_pos // 4, fast=32.0, slow=1.0))),
+               mlp=dict(kind="dense", ff=s["ff"]))
+    kinds = {
+        "A": att,
+        "M": dict(type="mlstm", mixer=dict(heads=s["m_heads"], dim=s["m_dim"], vdim=s["m_vdim"], gate_cap=15.0),
+                  mlp=dict(kind="dense", ff=s["ff"])),
+        "G": dict(type="mingru", mixer=dict(width=s["gru"]), mlp=dict(kind="dense", ff=s["ff"])),
+    }
+    layers = [json.loads(json.dumps(kinds[pattern[i % len(pattern)]])) for i in range(s["layers"])]
+    return dict(architecture="Bezutar", vocab=s["vocab"], width=s["width"], max_positions=max_pos,
+                norm=dict(eps=1e-6), streams=4, canon=dict(taps=4),
+                embedding=dict(bigram=dict(buckets=50021, mul_prev=31, mul_cur=17)), layers=layers)
+
+
+def _random_init(model, seed=0):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if p.dim() >= 2 and p.dtype != torch.float32:
+                fan_in = p.shape[-1]
+                p.copy_((torch.randn(p.shape, generator=g) * fan_in ** -0.5).to(p.dtype))
+            elif name.endswith("w_gates"):
+                p.copy_(torch.randn(p.shape, generator=g) * p.shape[-1] ** -0.5)
+            elif name.endswith("weight") and p.dim() == 2:      # canon taps
+                p.copy_(torch.randn(p.shape, generator=g) * 0.2)
+
+
+def _time(fn):
+    sync = torch.cuda.synchronize if torch.cuda.is_available() else (lambda: None)
+    sync()
+    t0 = time.perf_counter()
+    fn()
+    sync()
+    return time.perf_counter() - t0
+
+
+def run_bezutar(size, pattern, batch, isl, osl, device):
+    from megatron_amd.inference.engine import DynamicInferenceEngine
+    from megatron_amd.models.bezutar import BezutarConfig, BezutarModel
+
+    s = SIZES[size]
+    cfg = BezutarConfig.from_dict(bezutar_config(s, pattern, isl + osl + 64), dtype=torch.bfloat16)
+    with torch.device(device):
+        model = BezutarModel(cfg).eval()
+    _random_init(model)
+    page = 64
+    eng = DynamicInferenceEngine(model, num_blocks=batch * ((isl + osl) // page + 2), block_size=page,
+                                 max_batch=batch, device=device, use_hip_graphs=False,
+                                 enable_prefix_caching=False)
+    g = torch.Generator().manual_seed(1)
+    prompts = [torch.randint(0, s["vocab"], (isl,), generator=g).tolist() for _ in range(batch)]
+
+    def once():
+        reqs = [eng.open_request() for _ in range(batch)]
+        t_pre = _time(lambda: eng.forward_batch([(r, p) for r, p in zip(reqs, prompts)]))
+        toks = [[int(x)] for x in torch.randint(0, s["vocab"], (batch,), generator=g)]
+
+        def dec():
+            for _ in range(osl):
+                eng.forward_batch([(r, t) for r, t in zip(reqs, toks)])
+        t_dec = _time(dec)
+        for r in reqs:
+            eng.close_request(r)
+        return t_pre, t_dec
+
+    once()                      # warm-up (GEMM algorithm selection, allocator)
+    t_pre, t_dec = once()
+    n = sum(p.numel() for p in model.parameters())
+    return dict(model=f"bezutar[{pattern}]", size=size, params_m=round(n / 1e6, 1),
+                prefill_tok_s=round(batch * isl / t_pre, 1), decode_tok_s=round(batch * osl / t_dec, 1),
+                prefill_ms=round(1e3 * t_pre, 2), decode_ms_per_step=round(1e3 * t_dec / osl, 3))
+
+
+def run_gpt_mla(size, batch, isl, osl, device):
+    from megatron_amd.config import TransformerConfig
+    from megatron_amd.inference.engine import DynamicInferenceEngine
+    from megatron_amd.inference.sampling import SamplingParams
+    from megatron_amd.models.gpt import GPTModel
+    from megatron_amd.parallel import grid as G
+    from megatron_amd.parallel.random import model_parallel_seed
+
+    s = SIZES[size]
+    if not G.grid_initialized():
+        G.initialize_model_parallel(world_size=1, rank=0)
+    model_parallel_seed(1234)
+    cfg = TransformerConfig(
+        num_layers=s["layers"], hidden_size=s["width"], num_attention_heads=s["heads"],
+        ffn_hidden_size=s["ff"], vocab_size=s["vocab"], max_position_embeddings=isl + osl + 64, bf16=True,
+        multi_latent_attention=True, q_lora_rank=s["q_rank"], kv_lora_rank=s["kv_rank"],
+        qk_nope_head_dim=s["dim"], qk_rope_head_dim=s["rot"], v_head_dim=s["vdim"])
+    with torch.device(device):
+        model = GPTModel(cfg).eval()
+    page = 64
+    eng = DynamicInferenceEngine(model, num_blocks=batch * ((isl + osl) // page + 2), block_size=page,
+                                 max_batch=batch, max_prefill_tokens=isl, device=device,
+                                 use_hip_graphs=False, enable_prefix_caching=False)
+    g = torch.Generator().manual_seed(1)
+    prompts = [torch.randint(0, s["vocab"], (isl,), generator=g).tolist() for _ in range(batch)]
+    params = SamplingParams(max_tokens=osl + 1, greedy=True, stop_on_eod=False)
+
+    def once():
+        for p in prompts:
+            eng.add_request(p, params)
+
+        def pre():
+            for _ in range(batch):
+                eng.step()
+
+        def dec():
+            for _ in range(osl):
+                eng.step()
+        t_pre, t_dec = _time(pre), _time(dec)
+        eng.finished.clear()
+        assert not eng.has_work()
+        return t_pre, t_dec
+
+    once()
+    t_pre, t_dec = once()
+    n = sum(p.numel() for p in model.parameters())
+    return dict(model="gpt-mla", size=size, params_m=round(n / 1e6, 1),
+                prefill_tok_s=round(batch * isl / t_pre, 1), decode_tok_s=round(batch * osl / t_dec, 1),
+                prefill_ms=round(1e3 * t_pre, 2), decode_ms_per_step=round(1e3 * t_dec / osl, 3))
+
+
+def main(args) -> None:
+    assert torch.cuda.is_available(), "the serving comparison needs a GPU"
+    device = torch.device("cuda", 0)
+    torch.cuda.set_device(0)
+    for size in args.serve_sizes.split(","):
+        for pattern in args.serve_patterns.split(","):
+            r = run_bezutar(size, pattern, args.serve_batch, args.serve_isl, args.serve_osl, device)
+            r.update(batch=args.serve_batch, isl=args.serve_isl, osl=args.serve_osl, dtype="bf16", data="synthetic")
+            print(json.dumps(r), flush=True)
+            torch.cuda.empty_cache()
+        if not args.serve_skip_baseline:
+            r = run_gpt_mla(size, args.serve_batch, args.serve_isl, args.serve_osl, device)
+            r.update(batch=args.serve_batch, isl=args.serve_isl, osl=args.serve_osl, dtype="bf16", data="synthetic")
+            print(json.dumps(r), flush=True)
+            torch.cuda.empty_cache()

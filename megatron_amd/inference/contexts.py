@@ -424,6 +424,23 @@ class RaggedBatch:
     host_start: List[int] = None
     host_slots: List[int] = None
     host_tables: List[List[int]] = None
+    _tiles: Dict[int, torch.Tensor] = None
+
+    def row_tiles(self, heads: int, device, rows_per_tile: int = 64) -> torch.Tensor:
+        """Work list of the matrix-core attention kernel: one entry
+        (request, first row) per tile of ``rows_per_tile`` (token, head) rows,
+        rows numbered token-major inside each request.  Cached per head count
+        (every attention layer of a step shares it)."""
+        if self._tiles is None:
+            self._tiles = {}
+        t = self._tiles.get(heads)
+        if t is None:
+            work = []
+            for r in range(self.num_requests):
+                rows = (self.host_cu[r + 1] - self.host_cu[r]) * heads
+                work.extend((r, row0) for row0 in range(0, rows, rows_per_tile))
+            t = self._tiles[heads] = torch.as_tensor(work, dtype=torch.int32).reshape(-1, 2).to(device)
+        return t
 
 
 class HybridInferenceContext:

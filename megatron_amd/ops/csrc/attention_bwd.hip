@@ -469,7 +469,7 @@ __global__ __launch_bounds__(512, 2) void attn_bwd_dkv_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// v4 dkv design (round-3 target; see profiles/README.md measurements):
+// v4 dkv design (target design):
 //   The v3 combined 32-row attempt spills (2 accumulator sets = 128 VGPRs
 //   minimum is fine, but the A/B operand sets on top are not).  Plan:
 //   phase 1 unchanged (8 waves x 16 kv rows compute S^T/dP^T per 64-q tile);
@@ -1118,8 +1118,8 @@ std::vector<torch::Tensor> attn_bwd(torch::Tensor dout, torch::Tensor q, torch::
   static const bool force_v2 = getenv("MEGATRON_AMD_ATTN_BWD_V2") != nullptr;
   const bool use_v3_dq = !force_v2 && sq >= 256;
   // dv/dk split (v3) measured slower than the combined v2 dkv at s=4096
-  // (dk's global A-fragment reads thrash L1; see profiles/README.md round-2
-  // notes) - combined v2 stays the default, split kept for future work.
+  // (dk global A-fragment reads thrash L1) - combined v2 stays the default, split kept for future work.
+
   static const bool force_dkv_v3 = getenv("MEGATRON_AMD_ATTN_DKV_V3") != nullptr;
   const bool use_v3_dkv = force_dkv_v3 && !force_v2 && skv >= 256;
   dim3 grid_dq((sq + (use_v3_dq ? 255 : 127)) / (use_v3_dq ? 256 : 128), b * hq);

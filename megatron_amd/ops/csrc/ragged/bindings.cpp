@@ -25,6 +25,9 @@ torch::Tensor assemble_latent_q(torch::Tensor qa, torch::Tensor qr, torch::Tenso
 torch::Tensor latent_sink_attention(torch::Tensor q, torch::Tensor pool, int64_t rank, torch::Tensor sink,
                                     double scale, torch::Tensor tok_req, torch::Tensor tok_pos,
                                     torch::Tensor tables, int64_t bs);
+torch::Tensor latent_sink_attention_mfma(torch::Tensor q, torch::Tensor pool, int64_t rank, torch::Tensor sink,
+                                         double scale, torch::Tensor tiles, torch::Tensor cu, torch::Tensor start_pos,
+                                         torch::Tensor tables, int64_t bs, int64_t nsplit);
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("embed_tokens", &embed_tokens);
@@ -38,4 +41,5 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("latent_kv_store", &latent_kv_store);
   m.def("assemble_latent_q", &assemble_latent_q);
   m.def("latent_sink_attention", &latent_sink_attention);
+  m.def("latent_sink_attention_mfma", &latent_sink_attention_mfma);
 }

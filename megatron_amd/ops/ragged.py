@@ -147,8 +147,24 @@ def assemble_latent_q(q_abs, q_rot, cos, sin, rot_dims, batch):
     return torch.cat([q_abs, ref.rope_heads(q_rot, cos, sin, rot_dims, batch)], dim=-1)
 
 
+def _mfma_ok(q, rank) -> bool:
+    Dk = q.shape[2]
+    return (q.dtype == torch.bfloat16 and Dk % 8 == 0 and rank % 4 == 0 and Dk <= 576 and rank <= 512
+            and os.environ.get("MEGATRON_AMD_NO_MFMA_LATENT", "0") != "1")
+
+
 def latent_sink_attention(q, pool, rank, sink, scale, batch):
+    """[T, H, rank] (a view of an [H, T, rank] buffer on the kernel paths)."""
     if _native(q):
+        if _mfma_ok(q, rank):
+            # matrix-core kernel: 64 (token, head) rows per workgroup; steps with few
+            # rows and long contexts (decode) also split the keys over workgroups
+            tiles = batch.row_tiles(q.shape[1], q.device)
+            nblk = tiles.shape[0]
+            nsplit = max(1, min((batch.max_context + 127) // 128, 512 // nblk))
+            return _C.latent_sink_attention_mfma(q, pool, int(rank), sink, float(scale), tiles, batch.cu_tokens,
+                                                 batch.start_pos, batch.block_tables, int(batch.block_size),
+                                                 int(nsplit))
         return _C.latent_sink_attention(q, pool, int(rank), sink, float(scale), batch.tok_req,
                                         batch.tok_pos, batch.block_tables, int(batch.block_size))
     return ref.latent_sink_attention(q, pool, rank, sink, scale, batch)

@@ -146,7 +146,7 @@ class MambaMixer(nn.Module):
         # CP: the scan is sequential over the sequence, so CP shards are
         # gathered to the full sequence, scanned, and re-sliced (reference
         # mamba_context_parallel.py; this is the correct redundant-compute
-        # baseline — head-split CP is the round-2 optimization)
+        # baseline — head-split CP below is the optimization)
         cp = G.get_context_parallel_world_size()
         cp_mode = getattr(self.config, "cp_comm_type", "p2p")
         # head-split CP (reference MambaContextParallel intent, Ulysses-style):

@@ -8,7 +8,7 @@ part and a rotary (rope) part where k_rope is a single shared head.
 
 Default dims (nope 64 + rope 64 = 128 qk, v 128) keep the concatenated head
 dim inside the flash kernel's supported set; other dims fall back to the
-torch reference attention (absorbed-matmul inference path: round 2).
+torch reference attention (absorbed-matmul inference path).
 """
 
 from __future__ import annotations

@@ -37,6 +37,7 @@ RAGGED_SRC = [
     "megatron_amd/ops/csrc/ragged/streams.hip",
     "megatron_amd/ops/csrc/ragged/recurrent.hip",
     "megatron_amd/ops/csrc/ragged/latent_attention.hip",
+    "megatron_amd/ops/csrc/ragged/latent_attention_mfma.hip",
 ]
 
 # MEGATRON_AMD_ONLY_EXT=ragged builds just the serving kernels of the

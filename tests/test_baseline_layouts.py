@@ -3,7 +3,7 @@
 Each headline config's parallelism layout (TP=8; TP=4 x PP=2 interleaved;
 EP=8 all-to-all) runs on a tiny model at its real world size (8 CPU ranks),
 resharded from a single-process checkpoint, and must reproduce the
-single-process first-step loss.  This is the VERDICT round-1 item 6 gloo
+single-process first-step loss.  This is the gloo
 matrix: every RCCL call pattern the 8-GPU bench will issue (TP AR/AG/RS,
 PP p2p + interleaved schedule, EP a2a) exercised at the real group sizes.
 """

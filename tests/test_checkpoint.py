@@ -237,7 +237,7 @@ def test_moe_ep2_checkpoint_reshards_to_single(tmp_path):
     assert_close(out, ref["out"], rtol=1e-5, atol=1e-5)
 
 
-# --- round-2: windowed load + background-process async save -----------------
+# --- windowed load + background-process async save -----------------
 
 
 def test_windowed_load_does_not_assemble_full_tensors(tmp_path, monkeypatch):

@@ -302,7 +302,7 @@ def _run_mla_cp(rank, world, cfg_kwargs, tokens, labels, loss_ref, grad_ref, mod
 def test_mla_cp2_matches_single():
     """MLA training under CP=2 (ring p2p AND ulysses a2a) matches CP=1:
     global RoPE positions + LSE-merged ring partials on the unequal
-    dqk/dv head dims (closes the round-1 'MLA: CP not routed' limitation)."""
+    dqk/dv head dims."""
     cfg_kwargs = dict(num_layers=2, hidden_size=64, num_attention_heads=4,
                       num_query_groups=4, ffn_hidden_size=128, vocab_size=128,
                       max_position_embeddings=128, multi_latent_attention=True,

@@ -180,7 +180,7 @@ def test_rccl_registered_buffers_fallback_cpu():
         assert p_.main_grad is not None
 
 
-# --- expert-grad scaling + grad-norm group fixes (round-2 ADVICE items) -----
+# --- expert-grad scaling + grad-norm group fixes -----
 
 
 def _expert_scale_case(rank, world):

@@ -101,7 +101,7 @@ def test_tiny_mamba_loss_curve_matches_golden():
     _check_or_record("tiny_mamba.json", losses)
 
 
-# --- round-2: widened functional matrix (reference
+# --- widened functional matrix (reference
 # tests/functional_tests config-per-case pattern) ----------------------------
 
 
