@@ -160,7 +160,7 @@ def main(args) -> None:
     device = torch.device("cuda", 0)
     torch.cuda.set_device(0)
     for size in args.serve_sizes.split(","):
-        for pattern in args.serve_patterns.split(","):
+        for pattern in [p for p in args.serve_patterns.split(",") if p and p != "none"]:
             r = run_bezutar(size, pattern, args.serve_batch, args.serve_isl, args.serve_osl, device)
             r.update(batch=args.serve_batch, isl=args.serve_isl, osl=args.serve_osl, dtype="bf16", data="synthetic")
             print(json.dumps(r), flush=True)
