@@ -46,6 +46,32 @@ def _oracle_greedy(model, prompt, n_new):
     return out
 
 
+# bf16 logit noise between two correct attention paths (one flash pass over a
+# whole prompt vs portions over gathered pages vs one-token decode) on this
+# random-init model; top-2 margins of its logits are often below it
+TIE = 0.13
+
+
+def _assert_same_greedy_up_to_ties(model, prompt, a, b):
+    """Two greedy continuations must agree token for token until the first
+    place where they differ, and a difference is accepted only where the
+    no-cache reference itself is undecided: both tokens within TIE of its best
+    logit.  Past a tie the two are different (both valid) trajectories."""
+    toks = list(prompt)
+    for i, (x, y) in enumerate(zip(a, b)):
+        if x == y:
+            toks.append(x)
+            continue
+        with torch.no_grad():
+            lg = model(torch.tensor([toks], device="cuda"))[-1, 0].float()
+        best = float(lg.max())
+        assert best - float(lg[x]) <= TIE and best - float(lg[y]) <= TIE, (
+            f"token {i}: {x} vs {y} differ where the reference is decided "
+            f"(gaps {best - float(lg[x]):.3f}, {best - float(lg[y]):.3f})")
+        return
+    assert len(a) == len(b)
+
+
 def test_static_engine_gpu_matches_oracle(gpu_model):
     prompts = [[3, 7, 11, 2, 9, 100, 42], [5, 1]]
     eng = StaticInferenceEngine(gpu_model, max_batch=4, max_seq=256)
@@ -60,7 +86,11 @@ def test_dynamic_engine_gpu_matches_static(gpu_model):
     static = StaticInferenceEngine(gpu_model, max_batch=4, max_seq=256).generate(prompts, params)
     dynamic = DynamicInferenceEngine(gpu_model, num_blocks=32, block_size=16,
                                      max_prefill_tokens=16).generate(prompts, params)
-    for a, b in zip(static, dynamic):
+    for p, a, b in zip(prompts, static, dynamic):
+        _assert_same_greedy_up_to_ties(gpu_model, p, a.output_tokens, b.output_tokens)
+    # unchunked prefill takes the same flash pass as the static engine: exact
+    whole = DynamicInferenceEngine(gpu_model, num_blocks=32, block_size=16).generate(prompts, params)
+    for a, b in zip(static, whole):
         assert a.output_tokens == b.output_tokens
 
 
@@ -93,5 +123,5 @@ def test_speculative_decode_gpu_matches_plain(gpu_model):
 
     for draft_fn in (oracle_draft, lambda t: [0, 0], None):
         got = eng.generate_speculative(prompts, params, draft_fn=draft_fn, num_draft=3)
-        for a, b in zip(plain, got):
-            assert a.output_tokens == b.output_tokens
+        for p, a, b in zip(prompts, plain, got):
+            _assert_same_greedy_up_to_ties(gpu_model, p, a.output_tokens, b.output_tokens)
