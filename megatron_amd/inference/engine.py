@@ -756,6 +756,8 @@ class DynamicInferenceEngine:
             flat.extend(toks)
             rows.extend(base + w for w in (want[i] if want is not None else [n - 1]))
             base += n
+        if min(flat) < 0 or max(flat) >= self.model.config.vocab_size:
+            raise ValueError("token id outside the vocabulary")
         ctx.begin_batch(counts, starts, slots, tables)
         tokens = torch.as_tensor(flat, dtype=torch.long).to(self.device)
         for (req, toks), n in zip(feeds, counts):

@@ -54,6 +54,8 @@ def replay(engine, lines, out_dir: str, log=sys.stdout) -> None:
             req = live.get(e["id"])
             if req is None:
                 req = live[e["id"]] = engine.open_request()
+            if not e["tokens"]:
+                continue                    # admitted, nothing to run yet
             feeds.append((req, [int(t) for t in e["tokens"]]))
             want.append([int(w) for w in e.get("want", [])])
         logits = engine.forward_batch(feeds, want) if feeds else None

@@ -82,18 +82,31 @@ __global__ __launch_bounds__(256) void mlstm_kernel(
   const float qscale = 1.f / sqrtf((float)D);
   const float bih = bi[hd], bfh = bfg[hd];
   const int t0 = cu[r], t1 = cu[r + 1];
-  for (int t = t0; t < t1; ++t) {
+  // operands of the next token are fetched while the current one is processed:
+  // the recurrence is a serial chain, so global latency must not sit on it
+  float nq = 0.f, nk = 0.f, nv = 0.f, ngi = 0.f, ngf = 0.f;
+  auto fetch = [&](int t) {
     const T* row = qkvg + (long)t * stride;
-    for (int d = threadIdx.x; d < D; d += 256) {
-      sq[d] = ldf(row + hd * D + d) * qscale;
-      sk[d] = ldf(row + (long)H * D + hd * D + d);
+    if ((int)threadIdx.x < D) {
+      nq = ldf(row + hd * D + threadIdx.x) * qscale;
+      nk = ldf(row + (long)H * D + hd * D + threadIdx.x);
     }
     if (threadIdx.x < ML_VT) {
       const int cc = vt * ML_VT + threadIdx.x;
-      sv[threadIdx.x] = (cc < V) ? ldf(row + 2L * H * D + (long)hd * V + cc) : 0.f;
+      nv = (cc < V) ? ldf(row + 2L * H * D + (long)hd * V + cc) : 0.f;
     }
-    const float ig = cap * tanhf((gates[(long)t * 2 * H + hd] + bih) / cap);
-    const float fc = cap * tanhf((gates[(long)t * 2 * H + H + hd] + bfh) / cap);
+    ngi = gates[(long)t * 2 * H + hd];
+    ngf = gates[(long)t * 2 * H + H + hd];
+  };
+  if (t0 < t1) fetch(t0);
+  for (int t = t0; t < t1; ++t) {
+    sq[threadIdx.x] = nq;                      // D <= 256 = blockDim: one element per thread
+    sk[threadIdx.x] = nk;
+    if (threadIdx.x < ML_VT) sv[threadIdx.x] = nv;
+    const float gi = ngi, gf = ngf;
+    if (t + 1 < t1) fetch(t + 1);
+    const float ig = cap * tanhf((gi + bih) / cap);
+    const float fc = cap * tanhf((gf + bfh) / cap);
     const float fg = -softplusf_(-fc);               // log sigmoid
     const float mn = fmaxf(fg + m, ig);
     const float da = expf(fg + m - mn), db = expf(ig - mn);

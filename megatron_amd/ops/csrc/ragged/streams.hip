@@ -74,12 +74,14 @@ torch::Tensor embed_tokens(torch::Tensor tokens, torch::Tensor cu, torch::Tensor
 // ---------------------------------------------------------------------------
 constexpr int HC_MAX_STREAMS = 8;
 
-template <typename TY>
-__global__ __launch_bounds__(256) void hc_mix_norm_kernel(
+// BLOCK = 1024 for steps with few tokens (decode): one workgroup owns a token, so
+// more threads are the only way to have more loads in flight.
+template <typename TY, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void hc_mix_norm_kernel(
     float* __restrict__ streams, const TY* __restrict__ y, long y_stride, const float* __restrict__ mix,
     const float* __restrict__ out_w, const float* __restrict__ in_w, const float* __restrict__ norm_w,
     float eps, float* __restrict__ h, int S, int W) {
-  __shared__ float red[256 / WAVE];
+  __shared__ float red[BLOCK / WAVE];
   __shared__ float s_mix[HC_MAX_STREAMS * HC_MAX_STREAMS], s_out[HC_MAX_STREAMS], s_in[HC_MAX_STREAMS];
   const int t = blockIdx.x;
   if (threadIdx.x < S * S && y != nullptr) s_mix[threadIdx.x] = mix[threadIdx.x];
@@ -90,7 +92,7 @@ __global__ __launch_bounds__(256) void hc_mix_norm_kernel(
   __syncthreads();
   float* xs_base = streams + (long)t * S * W;
   float ss = 0.f;
-  for (int c = threadIdx.x; c < W; c += 256) {
+  for (int c = threadIdx.x; c < W; c += BLOCK) {
     float xs[HC_MAX_STREAMS];
 #pragma unroll
     for (int s = 0; s < HC_MAX_STREAMS; ++s) xs[s] = (s < S) ? xs_base[(long)s * W + c] : 0.f;
@@ -122,9 +124,9 @@ __global__ __launch_bounds__(256) void hc_mix_norm_kernel(
     }
   }
   if (in_w == nullptr) return;
-  const float total = block_reduce_sum<256>(ss, red);
+  const float total = block_reduce_sum<BLOCK>(ss, red);
   const float rs = rsqrtf(total / (float)W + eps);
-  for (int c = threadIdx.x; c < W; c += 256) {
+  for (int c = threadIdx.x; c < W; c += BLOCK) {
     const long i = (long)t * W + c;
     h[i] = h[i] * rs * (1.f + norm_w[c]);   // same thread wrote h[i] above
   }
@@ -155,15 +157,20 @@ torch::Tensor hc_mix_norm(torch::Tensor streams, torch::Tensor y, torch::Tensor 
   float* hp = has_in ? h.data_ptr<float>() : nullptr;
   const float* inp = has_in ? in_w.data_ptr<float>() : nullptr;
   const float* nwp = has_in ? norm_w.data_ptr<float>() : nullptr;
+  const bool wide = T_ < 512 && W >= 1024;
+#define HC_LAUNCH(TY, BLOCK, YP, YS, MP, OP)                                                              \
+  hipLaunchKernelGGL((hc_mix_norm_kernel<TY, BLOCK>), dim3(T_), dim3(BLOCK), 0, stream,                   \
+                     streams.data_ptr<float>(), YP, YS, MP, OP, inp, nwp, (float)eps, hp, S, W)
   if (has_y) {
-    RAGGED_DISPATCH(y, hipLaunchKernelGGL((hc_mix_norm_kernel<T>), dim3(T_), dim3(256), 0, stream,
-        streams.data_ptr<float>(), (const T*)y.data_ptr(), (long)y.stride(0), mix.data_ptr<float>(),
-        out_w.data_ptr<float>(), inp, nwp, (float)eps, hp, S, W));
+    RAGGED_DISPATCH(y, {
+      if (wide) HC_LAUNCH(T, 1024, (const T*)y.data_ptr(), (long)y.stride(0), mix.data_ptr<float>(), out_w.data_ptr<float>());
+      else HC_LAUNCH(T, 256, (const T*)y.data_ptr(), (long)y.stride(0), mix.data_ptr<float>(), out_w.data_ptr<float>());
+    });
   } else {
-    hipLaunchKernelGGL((hc_mix_norm_kernel<float>), dim3(T_), dim3(256), 0, stream, streams.data_ptr<float>(),
-                       (const float*)nullptr, 0L, (const float*)nullptr, (const float*)nullptr, inp, nwp,
-                       (float)eps, hp, S, W);
+    if (wide) HC_LAUNCH(float, 1024, (const float*)nullptr, 0L, (const float*)nullptr, (const float*)nullptr);
+    else HC_LAUNCH(float, 256, (const float*)nullptr, 0L, (const float*)nullptr, (const float*)nullptr);
   }
+#undef HC_LAUNCH
   return h;
 }
 

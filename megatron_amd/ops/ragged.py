@@ -161,7 +161,7 @@ def latent_sink_attention(q, pool, rank, sink, scale, batch):
             # rows and long contexts (decode) also split the keys over workgroups
             tiles = batch.row_tiles(q.shape[1], q.device)
             nblk = tiles.shape[0]
-            nsplit = max(1, min((batch.max_context + 127) // 128, 512 // nblk))
+            nsplit = max(1, min((batch.max_context + 63) // 64, 1024 // nblk, 64))
             return _C.latent_sink_attention_mfma(q, pool, int(rank), sink, float(scale), tiles, batch.cu_tokens,
                                                  batch.start_pos, batch.block_tables, int(batch.block_size),
                                                  int(nsplit))
