@@ -68,26 +68,28 @@ __global__ void assemble_q_kernel(const T* __restrict__ qa, long as_t, long as_h
                                   const float* __restrict__ sinv, int rot_dims, const int* __restrict__ tok_pos,
                                   T* __restrict__ out, int H, int rank, int rd) {
   const long t = blockIdx.x;
+  const int hd = blockIdx.y;
   const int Dk = rank + rd, half = rot_dims / 2;
   const long p = tok_pos[t];
-  for (int i = threadIdx.x; i < H * Dk; i += blockDim.x) {
-    const int hd = i / Dk, d = i % Dk;
+  const T* a = qa + t * as_t + hd * as_h;
+  const T* x = qr + t * rs_t + hd * rs_h;
+  T* dst = out + (t * H + hd) * Dk;
+  for (int d = threadIdx.x; d < Dk; d += blockDim.x) {
     float v;
     if (d < rank) {
-      v = ldf(qa + t * as_t + hd * as_h + d);
+      v = ldf(a + d);
     } else {
       const int e = d - rank;
-      const T* x = qr + t * rs_t + hd * rs_h;
       if (e < rot_dims) {
         const int j = (e < half) ? e : e - half;
         const float cs = cosv[p * half + j], sn = sinv[p * half + j];
-        const float a = ldf(x + j), b = ldf(x + j + half);
-        v = (e < half) ? (a * cs - b * sn) : (b * cs + a * sn);
+        const float u = ldf(x + j), w = ldf(x + j + half);
+        v = (e < half) ? (u * cs - w * sn) : (w * cs + u * sn);
       } else {
         v = ldf(x + e);
       }
     }
-    stf(out + t * (long)H * Dk + i, v);
+    stf(dst + d, v);
   }
 }
 
@@ -101,7 +103,7 @@ torch::Tensor assemble_latent_q(torch::Tensor qa, torch::Tensor qr, torch::Tenso
   auto out = torch::empty({T_, H, rank + rd}, qa.options());
   if (T_ == 0) return out;
   auto stream = at::cuda::getCurrentHIPStream();
-  RAGGED_DISPATCH(qa, hipLaunchKernelGGL((assemble_q_kernel<T>), dim3(T_), dim3(256), 0, stream,
+  RAGGED_DISPATCH(qa, hipLaunchKernelGGL((assemble_q_kernel<T>), dim3(T_, H), dim3(128), 0, stream,
       (const T*)qa.data_ptr(), (long)qa.stride(0), (long)qa.stride(1), (const T*)qr.data_ptr(),
       (long)qr.stride(0), (long)qr.stride(1), cosv.data_ptr<float>(), sinv.data_ptr<float>(), (int)rot_dims,
       tok_pos.data_ptr<int>(), (T*)out.data_ptr(), H, rank, rd));

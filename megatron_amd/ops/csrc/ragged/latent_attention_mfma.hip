@@ -148,18 +148,29 @@ __global__ __launch_bounds__(256) void latent_attn_mfma_kernel(
     __syncthreads();
     if (tile + 1 < tile_hi) issue(tile + 1);
     if (j0 <= kend_wave) {                        // wave-uniform: later tiles are all masked for this wave's rows
-      f32x4 st[2];
+      // two independent accumulation chains per key sub-tile (even / odd k steps):
+      // four MFMAs in flight instead of two dependent ones
+      f32x4 st[2], st2[2];
 #pragma unroll
       for (int kvt = 0; kvt < 2; ++kvt) {
         st[kvt] = f32x4{0.f, 0.f, 0.f, 0.f};
-        const short* krow = lds + (kvt * 16 + c) * ldk + 8 * g;
+        st2[kvt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      }
 #pragma unroll
-        for (int ks = 0; ks < NKS; ++ks) {
-          short8 tmp = *reinterpret_cast<const short8*>(krow + ks * 32);
-          st[kvt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<bf16x8*>(&tmp), qb[ks], st[kvt],
-                                                            0, 0, 0);
+      for (int ks = 0; ks < NKS; ++ks) {
+#pragma unroll
+        for (int kvt = 0; kvt < 2; ++kvt) {
+          short8 tmp = *reinterpret_cast<const short8*>(lds + (kvt * 16 + c) * ldk + 8 * g + ks * 32);
+          if (ks & 1)
+            st2[kvt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<bf16x8*>(&tmp), qb[ks], st2[kvt],
+                                                               0, 0, 0);
+          else
+            st[kvt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<bf16x8*>(&tmp), qb[ks], st[kvt],
+                                                              0, 0, 0);
         }
       }
+      st[0] += st2[0];
+      st[1] += st2[1];
       float s[8];
       bool ok[8];
       float mx = LA_NEG;

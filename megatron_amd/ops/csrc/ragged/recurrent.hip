@@ -58,14 +58,24 @@ torch::Tensor mingru_scan(torch::Tensor zxg, torch::Tensor bz, torch::Tensor bx,
 // reduced over row groups through LDS.
 // ---------------------------------------------------------------------------
 constexpr int ML_VT = 16, ML_RG = 16, ML_RPT = 16;   // dim <= RG * RPT = 256
+constexpr int ML_CH = 16;                             // tokens staged per chunk
 
+// Tokens are taken in chunks of ML_CH: q, k, the v tile and the gate
+// pre-activations of a whole chunk are loaded at once (one global latency per
+// chunk instead of one per token), the capped log gates are evaluated in
+// parallel (one thread per token) and the scalar stabiliser chain m, e^{f+m-m'},
+// e^{i-m'}, e^{-m'} is run once by one thread; the serial loop over the chunk
+// then only does the state update and the two reductions, with one barrier per
+// token (the reduction buffer is double-buffered).
 template <typename T>
 __global__ __launch_bounds__(256) void mlstm_kernel(
     const T* __restrict__ qkvg, long stride, const float* __restrict__ gates, const float* __restrict__ bi,
     const float* __restrict__ bfg, float* __restrict__ stS, float* __restrict__ stn, float* __restrict__ stm,
     const int* __restrict__ cu, const int* __restrict__ slots, float* __restrict__ o, int H, int D, int V,
     float cap) {
-  __shared__ float sq[ML_RG * ML_RPT], sk[ML_RG * ML_RPT], sv[ML_VT], red[ML_RG][ML_VT + 1];
+  __shared__ float sq[ML_CH][ML_RG * ML_RPT], sk[ML_CH][ML_RG * ML_RPT], sv[ML_CH][ML_VT];
+  __shared__ float s_ig[ML_CH], s_fg[ML_CH], s_da[ML_CH], s_db[ML_CH], s_em[ML_CH], s_m;
+  __shared__ float red[2][ML_RG][ML_VT + 1];
   const int r = blockIdx.x, hd = blockIdx.y, vt = blockIdx.z;
   const int c = threadIdx.x % ML_VT, rg = threadIdx.x / ML_VT;
   const int col = vt * ML_VT + c;
@@ -78,65 +88,73 @@ __global__ __launch_bounds__(256) void mlstm_kernel(
     S[i] = (row < D && colok) ? stS[((slot * H + hd) * D + row) * V + col] : 0.f;
     n[i] = (row < D) ? stn[(slot * H + hd) * D + row] : 0.f;
   }
-  float m = stm[slot * H + hd];
+  if (threadIdx.x == 0) s_m = stm[slot * H + hd];
   const float qscale = 1.f / sqrtf((float)D);
   const float bih = bi[hd], bfh = bfg[hd];
   const int t0 = cu[r], t1 = cu[r + 1];
-  // operands of the next token are fetched while the current one is processed:
-  // the recurrence is a serial chain, so global latency must not sit on it
-  float nq = 0.f, nk = 0.f, nv = 0.f, ngi = 0.f, ngf = 0.f;
-  auto fetch = [&](int t) {
-    const T* row = qkvg + (long)t * stride;
-    if ((int)threadIdx.x < D) {
-      nq = ldf(row + hd * D + threadIdx.x) * qscale;
-      nk = ldf(row + (long)H * D + hd * D + threadIdx.x);
-    }
-    if (threadIdx.x < ML_VT) {
-      const int cc = vt * ML_VT + threadIdx.x;
-      nv = (cc < V) ? ldf(row + 2L * H * D + (long)hd * V + cc) : 0.f;
-    }
-    ngi = gates[(long)t * 2 * H + hd];
-    ngf = gates[(long)t * 2 * H + H + hd];
-  };
-  if (t0 < t1) fetch(t0);
-  for (int t = t0; t < t1; ++t) {
-    sq[threadIdx.x] = nq;                      // D <= 256 = blockDim: one element per thread
-    sk[threadIdx.x] = nk;
-    if (threadIdx.x < ML_VT) sv[threadIdx.x] = nv;
-    const float gi = ngi, gf = ngf;
-    if (t + 1 < t1) fetch(t + 1);
-    const float ig = cap * tanhf((gi + bih) / cap);
-    const float fc = cap * tanhf((gf + bfh) / cap);
-    const float fg = -softplusf_(-fc);               // log sigmoid
-    const float mn = fmaxf(fg + m, ig);
-    const float da = expf(fg + m - mn), db = expf(ig - mn);
-    m = mn;
-    __syncthreads();
-    const float vv = sv[c];
-    float part = 0.f, npart = 0.f;
-#pragma unroll
-    for (int i = 0; i < ML_RPT; ++i) {
-      const int rr = rg + i * ML_RG;
-      if (rr < D) {
-        const float kk = sk[rr], qq = sq[rr];
-        S[i] = da * S[i] + db * kk * vv;
-        n[i] = da * n[i] + db * kk;
-        part += S[i] * qq;
-        npart += n[i] * qq;
+  int step = 0;
+  for (int tc = t0; tc < t1; tc += ML_CH) {
+    const int nc = min(ML_CH, t1 - tc);
+    if ((int)threadIdx.x < D) {                  // D <= 256 = blockDim: one q and one k element per thread and token
+#pragma unroll 4
+      for (int tt = 0; tt < nc; ++tt) {
+        const T* row = qkvg + (long)(tc + tt) * stride;
+        sq[tt][threadIdx.x] = ldf(row + hd * D + threadIdx.x) * qscale;
+        sk[tt][threadIdx.x] = ldf(row + (long)H * D + hd * D + threadIdx.x);
       }
     }
-    red[rg][c] = part;
-    if (c == 0) red[rg][ML_VT] = npart;
-    __syncthreads();
-    if (rg == 0 && colok) {
-      float num = 0.f, nq = 0.f;
-#pragma unroll
-      for (int g = 0; g < ML_RG; ++g) {
-        num += red[g][c];
-        nq += red[g][ML_VT];
-      }
-      o[((long)t * H + hd) * V + col] = num / (fmaxf(fabsf(nq), expf(-m)) + 1e-6f);
+    {
+      const int tt = threadIdx.x / ML_VT, cc = vt * ML_VT + threadIdx.x % ML_VT;   // 16 x 16 = 256 threads
+      if (tt < nc) sv[tt][threadIdx.x % ML_VT] = (cc < V) ? ldf(qkvg + (long)(tc + tt) * stride + 2L * H * D + (long)hd * V + cc) : 0.f;
     }
+    if ((int)threadIdx.x < nc) {
+      const long t = tc + threadIdx.x;
+      s_ig[threadIdx.x] = cap * tanhf((gates[t * 2 * H + hd] + bih) / cap);
+      const float fc = cap * tanhf((gates[t * 2 * H + H + hd] + bfh) / cap);
+      s_fg[threadIdx.x] = -softplusf_(-fc);      // log sigmoid
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      float mm = s_m;
+      for (int tt = 0; tt < nc; ++tt) {
+        const float mn = fmaxf(s_fg[tt] + mm, s_ig[tt]);
+        s_da[tt] = expf(s_fg[tt] + mm - mn);
+        s_db[tt] = expf(s_ig[tt] - mn);
+        s_em[tt] = expf(-mn);
+        mm = mn;
+      }
+      s_m = mm;
+    }
+    __syncthreads();
+    for (int tt = 0; tt < nc; ++tt, ++step) {
+      const float da = s_da[tt], db = s_db[tt], vv = sv[tt][c];
+      float part = 0.f, npart = 0.f;
+#pragma unroll
+      for (int i = 0; i < ML_RPT; ++i) {
+        const int rr = rg + i * ML_RG;
+        if (rr < D) {
+          const float kk = sk[tt][rr], qq = sq[tt][rr];
+          S[i] = da * S[i] + db * kk * vv;
+          n[i] = da * n[i] + db * kk;
+          part += S[i] * qq;
+          npart += n[i] * qq;
+        }
+      }
+      float(*rb)[ML_VT + 1] = red[step & 1];
+      rb[rg][c] = part;
+      if (c == 0) rb[rg][ML_VT] = npart;
+      __syncthreads();
+      if (rg == 0 && colok) {
+        float num = 0.f, nq = 0.f;
+#pragma unroll
+        for (int g = 0; g < ML_RG; ++g) {
+          num += rb[g][c];
+          nq += rb[g][ML_VT];
+        }
+        o[((long)(tc + tt) * H + hd) * V + col] = num / (fmaxf(fabsf(nq), s_em[tt]) + 1e-6f);
+      }
+    }
+    __syncthreads();                             // the chunk buffers are rewritten next
   }
 #pragma unroll
   for (int i = 0; i < ML_RPT; ++i) {
@@ -146,7 +164,7 @@ __global__ __launch_bounds__(256) void mlstm_kernel(
       if (vt == 0 && c == 0) stn[(slot * H + hd) * D + row] = n[i];
     }
   }
-  if (vt == 0 && threadIdx.x == 0) stm[slot * H + hd] = m;
+  if (vt == 0 && threadIdx.x == 0) stm[slot * H + hd] = s_m;
 }
 
 // per-head RMS norm of o, learned weight, sigmoid output gate; one wave per (token, head)
