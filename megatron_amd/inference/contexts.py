@@ -450,7 +450,10 @@ class HybridInferenceContext:
     * ``cache_specs``: name -> row width.  One paged pool per name,
       ``[num_blocks * block_size, width]`` in the compute dtype, addressed by the
       request's block table (all pools share the table: one page id covers
-      the same token range in every pool).
+      the same token range in every pool).  A value ``(width, rows_per_page)``
+      makes a pool with fewer rows a page, for caches that hold one row per
+      group of tokens (pooled keys): entry e of a request lives in its page
+      ``e // rows_per_page`` at offset ``e % rows_per_page``.
     * ``state_specs``: name -> (per-slot shape, dtype).  One tensor per name,
       ``[num_slots, *shape]``; recurrent state is kept in 32-bit floats whatever
       the compute dtype.
@@ -467,8 +470,12 @@ class HybridInferenceContext:
         self.compute_dtype = dtype
         self.allocator = KVBlockAllocator(num_blocks, first_id=0)
         self.slot_allocator = StateSlotAllocator(num_slots)
-        self.pools = {name: torch.zeros(num_blocks * block_size, width, dtype=dtype, device=device)
-                      for name, width in cache_specs.items()}
+        self.pools = {}
+        for name, width in cache_specs.items():
+            per_page = block_size
+            if isinstance(width, (tuple, list)):
+                width, per_page = width
+            self.pools[name] = torch.zeros(num_blocks * per_page, width, dtype=dtype, device=device)
         self.states = {name: torch.zeros(num_slots, *shape, dtype=sdt, device=device)
                        for name, (shape, sdt) in state_specs.items()}
         self.batch: Optional[RaggedBatch] = None

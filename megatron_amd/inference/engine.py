@@ -403,7 +403,7 @@ class DynamicInferenceEngine:
         # prompts beside single decoded tokens in ONE forward per step
         self.ragged = bool(getattr(model, "ragged_batch", False))
         if self.ragged:
-            spec = model.inference_spec()
+            spec = model.inference_spec(block_size)
             self.context = HybridInferenceContext(
                 spec.caches, spec.states, num_blocks=num_blocks, block_size=block_size,
                 num_slots=max_batch, dtype=cfg.params_dtype, device=device)
@@ -745,7 +745,8 @@ class DynamicInferenceEngine:
         for i, (req, toks) in enumerate(feeds):
             n = len(toks)
             assert n > 0, "a feed brings at least one token"
-            if req.cached + n > self.model.config.max_position_embeddings:
+            limit = getattr(self.model.config, "max_position_embeddings", None)
+            if limit is not None and req.cached + n > limit:
                 raise RuntimeError("request exceeds the model's position range")
             if not self._ensure_blocks(req, req.cached + n):
                 raise RuntimeError("cache pool exhausted")

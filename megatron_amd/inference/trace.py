@@ -87,14 +87,14 @@ def main(argv=None) -> int:
     ap.add_argument("--device", default=None)
     a = ap.parse_args(argv)
     device = torch.device(a.device) if a.device else None
-    if (device is None and torch.cuda.is_available()) or (device is not None and device.type == "cuda"):
-        from megatron_amd.ops import ragged
-
-        if ragged._C is None:
-            print("building the ragged-ops extension (first call)", file=sys.stderr, flush=True)
-            ragged.build_ragged_ops()
     dtype = torch.bfloat16 if a.dtype == "bfloat16" else torch.float32
     engine = build_engine(a.model, dtype, a.max_tokens, device)
+    if engine.device.type == "cuda":
+        # kernels are compiled in-tree at the first call, and only the
+        # extensions this model's layers use
+        from megatron_amd.ops import ragged
+
+        ragged.ensure_built(getattr(engine.model, "native_extensions", ("ragged",)), verbose=True)
     os.makedirs(a.out, exist_ok=True)
     replay(engine, sys.stdin, a.out)
     return 0

@@ -23,4 +23,8 @@ def __getattr__(name):  # lazy: bert/t5/llava/audio pull heavier deps
         from megatron_amd.models import bezutar
 
         return getattr(bezutar, name)
+    if name in ("BezuraxModel", "BezuraxConfig"):
+        from megatron_amd.models import bezurax
+
+        return getattr(bezurax, name)
     raise AttributeError(name)

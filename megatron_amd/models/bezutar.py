@@ -64,7 +64,9 @@ class BezutarConfig:
 
 @dataclass
 class InferenceSpec:
-    """What a model asks of the cache/state manager."""
+    """What a model asks of the cache/state manager: paged pools (name -> row
+    width, or (row width, rows a page) for pools that hold fewer rows than
+    tokens) and per-request state tensors (name -> (shape, dtype))."""
 
     caches: Dict[str, int]
     states: Dict[str, tuple]
@@ -145,7 +147,7 @@ class BezutarModel(nn.Module):
 
     # -- what the cache/state manager must provide ------------------------------
 
-    def inference_spec(self) -> InferenceSpec:
+    def inference_spec(self, page: int = 64) -> InferenceSpec:
         caches, states = {}, {}
         for layer in self.layers:
             caches.update(layer.mixer.cache_spec())

@@ -52,6 +52,13 @@ def _bezutar(path, dtype, device):
     return build_bezutar_from_dir(path, dtype=dtype, device=device)
 
 
+@register_model("Bezurax")
+def _bezurax(path, dtype, device):
+    from megatron_amd.models.bezurax import build_bezurax_from_dir
+
+    return build_bezurax_from_dir(path, dtype=dtype, device=device)
+
+
 @register_model("LlamaForCausalLM")
 def _llama(path, dtype, device):
     """HuggingFace Llama checkpoints -> GPTModel (single process, TP=1)."""

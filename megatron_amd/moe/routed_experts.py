@@ -1,0 +1,79 @@
+"""Routed clamped-GLU experts for the ragged serving path (single process, all
+experts resident; the training-side MoE with token dispatchers is
+moe/moe_layer.py).
+
+Router: logits in fp32, sigmoid scores, the ``top`` largest among the experts
+of the best ``keep`` of ``groups`` neighbour groups (group score = sum of its
+two largest scores; the selection rule of moe/router.py::group_limited_topk),
+weights = chosen scores / their sum * route_scale.
+Expert (no biases): g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit),
+y = g sigmoid(alpha g) (u + 1), output W_down y.
+Optional shared expert of the same form for every token, times
+sigmoid(w_sg . h); its gate row rides in the fp32 router GEMM.
+
+Step: one fp32 GEMM [router; shared gate], a routing kernel, then the
+(token, choice) pairs are sorted by expert and each expert with work runs its
+gate/up and down products on its slice (vendor GEMMs; the pair counts are the
+step's one host read), and one kernel forms
+sum_k weight_k down_k + sigmoid(gate) shared + add in fp32.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from megatron_amd.ops import ragged as R
+
+
+class RoutedExpertsMLP(nn.Module):
+    def __init__(self, hidden: int, experts: int, top: int, ff: int, limit: float, groups: int = 1,
+                 keep: int = 1, route_scale: float = 1.0, shared_ff: Optional[int] = None,
+                 shared_limit: Optional[float] = None, alpha: float = 1.702, dtype=torch.bfloat16):
+        super().__init__()
+        assert top <= experts and experts % max(groups, 1) == 0
+        if groups > 1:
+            assert keep * (experts // groups) >= top, "the kept groups hold fewer experts than are chosen"
+        self.experts, self.top, self.ff, self.limit = experts, top, ff, float(limit)
+        self.groups, self.keep, self.route_scale, self.alpha = max(groups, 1), keep, float(route_scale), float(alpha)
+        self.shared_ff = shared_ff
+        self.shared_limit = float(shared_limit) if shared_ff else None
+        # row ``experts`` (when there is a shared expert) is its gate vector
+        self.w_router = nn.Parameter(torch.zeros(experts + (1 if shared_ff else 0), hidden, dtype=torch.float32))
+        self.w_gate_up = nn.Parameter(torch.zeros(experts, 2 * ff, hidden, dtype=dtype))   # [gate; up] per expert
+        self.w_down = nn.Parameter(torch.zeros(experts, hidden, ff, dtype=dtype))
+        if shared_ff:
+            self.ws_gate_up = nn.Parameter(torch.zeros(2 * shared_ff, hidden, dtype=dtype))
+            self.ws_down = nn.Parameter(torch.zeros(hidden, shared_ff, dtype=dtype))
+
+    def route(self, h: torch.Tensor):
+        logits = F.linear(h.float(), self.w_router)
+        ids, weights = R.moe_route(logits, self.experts, self.top, self.groups, self.keep, self.route_scale)
+        return logits, ids, weights
+
+    def forward(self, h: torch.Tensor, add: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """h [T, hidden] in the compute dtype -> fp32 [T, hidden] (+ add)."""
+        T, K, E = h.shape[0], self.top, self.experts
+        logits, ids, weights = self.route(h)
+        flat = ids.reshape(-1).long()
+        order = torch.argsort(flat, stable=True)              # pairs sorted by expert
+        inv = torch.empty_like(order)
+        inv[order] = torch.arange(order.numel(), device=order.device)
+        counts = torch.bincount(flat, minlength=E).tolist()   # the step's host read
+        xs = h.index_select(0, torch.div(order, K, rounding_mode="floor"))
+        down = torch.empty(T * K, h.shape[1], dtype=h.dtype, device=h.device)
+        at = 0
+        for e, n in enumerate(counts):
+            if n:
+                gu = F.linear(xs[at:at + n], self.w_gate_up[e])
+                down[at:at + n] = F.linear(R.clamped_glu(gu, self.limit, self.alpha, h.dtype), self.w_down[e])
+                at += n
+        shared = gate = None
+        if self.shared_ff:
+            sy = R.clamped_glu(F.linear(h, self.ws_gate_up), self.shared_limit, self.alpha, h.dtype)
+            shared = F.linear(sy, self.ws_down)
+            gate = logits[:, E].contiguous()
+        return R.moe_combine(down, inv.view(T, K).to(torch.int32), weights, shared, gate, add)

@@ -20,40 +20,66 @@ import torch
 from megatron_amd.ops import ragged_reference as ref
 from megatron_amd.ops.ragged_reference import rope_table  # noqa: F401  (host-side table)
 
-_C = None
+_C = None      # _ragged_ops: latent attention, mLSTM, minGRU, hyper-connections, canon conv, xIELU
+_H = None      # _hybrid_ops: grouped norm, pooled-window attention, delta rule, routed experts
 _IMPORT_ERROR: Optional[str] = None
+_IMPORT_ERRORS = {}
+
+# setup.py extension key -> module name; a model names the keys it needs in
+# ``native_extensions`` and a serving process builds only those on first use
+EXTENSIONS = {"ragged": "_ragged_ops", "hybrid": "_hybrid_ops"}
 
 
-def _load():
-    global _C, _IMPORT_ERROR
-    if _C is not None:
-        return _C
+def _load(key: str = "ragged"):
+    global _C, _H, _IMPORT_ERROR
+    cur = _C if key == "ragged" else _H
+    if cur is not None:
+        return cur
     try:
-        from megatron_amd.ops import _ragged_ops as mod  # built in-tree (setup.py / build_ragged_ops)
+        import importlib
 
-        _C = mod
+        mod = importlib.import_module("megatron_amd.ops." + EXTENSIONS[key])  # built in-tree (setup.py)
+        if key == "ragged":
+            _C = mod
+        else:
+            _H = mod
+        return mod
     except Exception as e:  # noqa: BLE001
-        _IMPORT_ERROR = repr(e)
-    return _C
+        _IMPORT_ERRORS[key] = repr(e)
+        if key == "ragged":
+            _IMPORT_ERROR = repr(e)
+    return None
 
 
-_load()
+_load("ragged")
+_load("hybrid")
 
 
-def build_ragged_ops(verbose: bool = False) -> None:
-    """Compile ONLY the ragged-ops extension in-tree (a serving process of a
-    model that needs nothing else calls this on first use)."""
+def build_extension(key: str, verbose: bool = False) -> None:
+    """Compile ONE serving extension in-tree (a serving process of a model that
+    needs nothing else calls this on first use)."""
     import subprocess
     import sys
 
     repo = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
-    env = dict(os.environ, MEGATRON_AMD_ONLY_EXT="ragged", PYTORCH_ROCM_ARCH="gfx950")
+    env = dict(os.environ, MEGATRON_AMD_ONLY_EXT=key, PYTORCH_ROCM_ARCH="gfx950")
     env.setdefault("MAX_JOBS", "8")
     out = None if verbose else subprocess.DEVNULL
     subprocess.run([sys.executable, "setup.py", "build_ext", "--inplace"], cwd=repo, env=env,
                    check=True, stdout=sys.stderr if verbose else out, stderr=sys.stderr if verbose else out)
-    if _load() is None:
-        raise RuntimeError(f"ragged ops extension did not import after build: {_IMPORT_ERROR}")
+    if _load(key) is None:
+        raise RuntimeError(f"{EXTENSIONS[key]} did not import after build: {_IMPORT_ERRORS.get(key)}")
+
+
+def build_ragged_ops(verbose: bool = False) -> None:
+    build_extension("ragged", verbose)
+
+
+def ensure_built(keys, verbose: bool = False) -> None:
+    """Build the named extensions that are not there yet."""
+    for key in keys:
+        if _load(key) is None:
+            build_extension(key, verbose)
 
 
 def has_native() -> bool:
@@ -69,6 +95,16 @@ def _native(x: torch.Tensor) -> bool:
         raise RuntimeError(
             "megatron_amd ragged-ops HIP extension not built but a GPU tensor hit the ops layer "
             f"(import error: {_IMPORT_ERROR}). Run megatron_amd.ops.ragged.build_ragged_ops().")
+    return True
+
+
+def _native_h(x: torch.Tensor) -> bool:
+    if not x.is_cuda or os.environ.get("MEGATRON_AMD_FORCE_REFERENCE", "0") == "1":
+        return False
+    if _H is None:
+        raise RuntimeError(
+            "megatron_amd hybrid-ops HIP extension not built but a GPU tensor hit the ops layer "
+            f"(import error: {_IMPORT_ERRORS.get('hybrid')}). Run megatron_amd.ops.ragged.build_extension('hybrid').")
     return True
 
 
@@ -180,3 +216,85 @@ def gate_heads(x, gate_pre, heads):
     if _native(x):
         return _C.gate_heads(x, gate_pre, int(heads))
     return ref.gate_heads(x, gate_pre, heads)
+
+
+# ---------------------------------------------------------------------------
+# ops of the hybrid extension: plain fp32 residual with grouped RMS norm,
+# attention over a sliding window plus mean-pooled blocks, generalized delta
+# rule, routed clamped-GLU experts
+# ---------------------------------------------------------------------------
+
+
+def embed_plain(tokens, embed):
+    if _native_h(embed):
+        return _H.embed_plain(tokens, embed)
+    return ref.embed_plain(tokens, embed)
+
+
+def residual_group_norm(x, y, w_a, w_b, groups, eps, out_dtype):
+    """x fp32 [T, W] += y in place (y may be None); -> (norm(x) w_a, norm(x) w_b or None)."""
+    if _native_h(x):
+        d = x.device
+        h_a, h_b = _H.residual_group_norm(x, y if y is not None else _none(d), w_a,
+                                          w_b if w_b is not None else _none(d), int(groups), float(eps),
+                                          out_dtype == torch.bfloat16)
+        return h_a, (h_b if w_b is not None else None)
+    return ref.residual_group_norm(x, y, w_a, w_b, groups, eps, out_dtype)
+
+
+def qk_norm_store(proj, q_off, q_width, k_off, k_width, v_off, v_width, q_norm, k_norm, eps, pool, batch):
+    if _native_h(proj):
+        return _H.qk_norm_store(proj, int(q_off), int(q_width), int(k_off), int(k_width), int(v_off), int(v_width),
+                                q_norm, k_norm, float(eps), pool, batch.tok_row)
+    return ref.qk_norm_store(proj, q_off, q_width, k_off, k_width, v_off, v_width, q_norm, k_norm, eps, pool, batch)
+
+
+def pool_blocks(pool, pooled, block, pooled_per_page, batch):
+    if _native_h(pool):
+        _H.pool_blocks(pool, pooled, int(block), int(pooled_per_page), batch.cu_tokens, batch.start_pos,
+                       batch.block_tables, int(batch.block_size), int(batch.max_new))
+        return
+    ref.pool_blocks(pool, pooled, block, pooled_per_page, batch)
+
+
+def pooled_window_attention(q, pool, pooled, heads, kv_heads, dim, vdim, scale, window, block,
+                            pooled_per_page, batch, out, out_col, out_scale):
+    if _native_h(q):
+        _H.pooled_window_attention(q, pool, pooled, int(heads), int(kv_heads), int(dim), int(vdim), float(scale),
+                                   int(window), int(block), int(pooled_per_page), batch.tok_req, batch.tok_pos,
+                                   batch.block_tables, int(batch.block_size), out, int(out_col), float(out_scale))
+        return
+    ref.pooled_window_attention(q, pool, pooled, heads, kv_heads, dim, vdim, scale, window, block,
+                                pooled_per_page, batch, out, out_col, out_scale)
+
+
+def delta_rule_scan(proj, r_off, k_off, v_off, g_off, a_off, w_off, w_rank, w2, w0, a_bias, norm_w,
+                    heads, dim, eps, state, batch, out, out_col, out_scale):
+    if _native_h(proj):
+        _H.delta_rule_scan(proj, int(r_off), int(k_off), int(v_off), int(g_off), int(a_off), int(w_off),
+                           int(w_rank), w2, w0, a_bias, norm_w, int(heads), int(dim), float(eps), state,
+                           batch.cu_tokens, batch.slots, out, int(out_col), float(out_scale))
+        return
+    ref.delta_rule_scan(proj, r_off, k_off, v_off, g_off, a_off, w_off, w_rank, w2, w0, a_bias, norm_w,
+                        heads, dim, eps, state, batch, out, out_col, out_scale)
+
+
+def moe_route(logits, experts, top, groups, keep, scale):
+    if _native_h(logits):
+        return _H.moe_route(logits, int(experts), int(top), int(groups), int(keep), float(scale))
+    return ref.moe_route(logits, experts, top, groups, keep, scale)
+
+
+def clamped_glu(gu, limit, alpha, out_dtype):
+    if _native_h(gu):
+        return _H.clamped_glu(gu, float(limit), float(alpha))
+    return ref.clamped_glu(gu, limit, alpha, out_dtype)
+
+
+def moe_combine(down, inv, weights, shared, shared_gate, add):
+    if _native_h(down):
+        d = down.device
+        return _H.moe_combine(down, inv, weights, shared if shared is not None else _none(d),
+                              shared_gate if shared is not None else _none(d),
+                              add if add is not None else _none(d))
+    return ref.moe_combine(down, inv, weights, shared, shared_gate, add)

@@ -230,3 +230,174 @@ def gate_heads(x, gate_pre, heads):
     T = x.shape[0]
     g = torch.sigmoid(gate_pre.float())
     return (x.float() * g[:, :, None]).reshape(T, -1).to(x.dtype)
+
+
+# ---------------------------------------------------------------------------
+# grouped RMS norm on a plain fp32 residual, attention over a sliding window
+# plus mean-pooled blocks, generalized delta rule, routed clamped-GLU experts
+# ---------------------------------------------------------------------------
+
+
+def embed_plain(tokens, embed):
+    """x[t] = embed[tok] in fp32."""
+    return embed[tokens].float()
+
+
+def residual_group_norm(x, y, w_a, w_b, groups, eps, out_dtype):
+    """x [T, W] fp32 <- x + y (in place, when ``y`` is given), then RMS norm in
+    ``groups`` equal consecutive parts (each divided by its own root mean square)
+    times a plain weight; one normed copy per weight given (w_b may be None)."""
+    if y is not None:
+        x.add_(y.float())
+    T, W = x.shape
+    p = x.view(T, groups, W // groups)
+    n = (p * torch.rsqrt((p * p).mean(-1, keepdim=True) + eps)).reshape(T, W)
+    h_a = (n * w_a.float()).to(out_dtype)
+    h_b = (n * w_b.float()).to(out_dtype) if w_b is not None else None
+    return h_a, h_b
+
+
+def qk_norm_store(proj, q_off, q_width, k_off, k_width, v_off, v_width, q_norm, k_norm, eps, pool, batch):
+    """From the fused projection rows ``proj`` [T, *]: RMS norm of the whole query
+    slice (all heads at once) and of the whole key slice with plain weights;
+    the cache row of each token becomes [normed keys | values], the values
+    being the slice at ``v_off`` as projected.  Returns the normed queries."""
+    def norm(z, w):
+        z = z.float()
+        return z * torch.rsqrt((z * z).mean(-1, keepdim=True) + eps) * w.float()
+    q = norm(proj[:, q_off:q_off + q_width], q_norm).to(proj.dtype)
+    k = norm(proj[:, k_off:k_off + k_width], k_norm)
+    pool[batch.tok_row] = torch.cat([k, proj[:, v_off:v_off + v_width].float()], dim=-1).to(pool.dtype)
+    return q
+
+
+def _rows_of(table, n, per_page, device):
+    """cache rows of a request's entries 0..n-1 in a pool with per_page rows a page"""
+    idx = torch.arange(n, device=device)
+    return table[idx // per_page] * per_page + idx % per_page
+
+
+def pool_blocks(pool, pooled, block, pooled_per_page, batch):
+    """Mean of every block of ``block`` consecutive cache rows that this step
+    completed (its last position was written now), as the cache holds them,
+    into the pooled pool (entry b of a request = block b)."""
+    bs = batch.block_size
+    for r, a, b, start, slot in _spans(batch):
+        first, last = start // block, (start + b - a) // block
+        if last <= first:
+            continue
+        table = torch.as_tensor(batch.host_tables[r], dtype=torch.long, device=pool.device)
+        rows = _rows_of(table, last * block, bs, pool.device)[first * block:]
+        mean = pool[rows].float().view(last - first, block, -1).mean(1)
+        prow = _rows_of(table, last, pooled_per_page, pool.device)[first:]
+        pooled[prow] = mean.to(pooled.dtype)
+
+
+def pooled_window_attention(q, pool, pooled, heads, kv_heads, dim, vdim, scale, window, block,
+                            pooled_per_page, batch, out, out_col, out_scale):
+    """Grouped-query softmax attention over the paged cache where position i sees
+    the tokens j with 0 <= i - j < window and, beside them, one mean-pooled
+    key/value for each block of ``block`` tokens that ends at or before
+    i - window.  Cache rows are [kv_heads * dim keys | kv_heads * vdim values].
+    Writes out[:, out_col : out_col + heads * vdim] = out_scale * result."""
+    T = q.shape[0]
+    H, G, D, V = heads, kv_heads, dim, vdim
+    rep = H // G
+    bs = batch.block_size
+    dev = q.device
+    for r, a, b, start, slot in _spans(batch):
+        n = b - a
+        L = start + n
+        table = torch.as_tensor(batch.host_tables[r], dtype=torch.long, device=dev)
+        kv = pool[_rows_of(table, L, bs, dev)].float()
+        nb_max = max(0, L - window) // block
+        if nb_max > 0:
+            pk = pooled[_rows_of(table, nb_max, pooled_per_page, dev)].float()
+            kv = torch.cat([pk, kv], dim=0)
+        keys = kv[:, :G * D].view(-1, G, D)
+        vals = kv[:, G * D:].view(-1, G, V)
+        qi = torch.arange(start, L, device=dev)
+        j = torch.arange(L, device=dev)
+        tok_ok = (j[None, :] <= qi[:, None]) & (qi[:, None] - j[None, :] < window)
+        nb = torch.clamp(qi - window + 1, min=0) // block
+        blk_ok = torch.arange(nb_max, device=dev)[None, :] < nb[:, None]
+        ok = torch.cat([blk_ok, tok_ok], dim=1)                       # [n, nb_max + L]
+        qq = q[a:b].float().view(n, G, rep, D)
+        s = torch.einsum("ngrd,lgd->ngrl", qq, keys) * scale
+        s = s.masked_fill(~ok[:, None, None, :], float("-inf"))
+        p = torch.softmax(s, dim=-1)
+        o = torch.einsum("ngrl,lgv->ngrv", p, vals).reshape(n, H * V)
+        out[a:b, out_col:out_col + H * V] = (o * out_scale).to(out.dtype)
+
+
+def delta_rule_scan(proj, r_off, k_off, v_off, g_off, a_off, w_off, w_rank, w2, w0, a_bias, norm_w,
+                    heads, dim, eps, state, batch, out, out_col, out_scale):
+    """Generalized delta rule over a ragged batch.  ``proj`` [T, *] holds, at the
+    given column offsets, r, k, v, the output-gate and removal-rate
+    pre-activations (heads * dim each) and the decay bottleneck (w_rank).
+        decay   w = exp(-e^{-1/2} sigmoid(w2 tanh(.) + w0)),   removal a = sigmoid(. + a_bias)
+        unit key u = k / sqrt(sum k^2 + 1e-6)  (per head)
+        S <- diag(w) S - (a u)(u^T S) + k v^T  (both terms read the old S),  o = S^T r
+    Each head's o is divided by its root mean square, times norm_w, times
+    sigmoid(gate).  state [slots, heads, dim, dim] fp32.  Writes
+    out[:, out_col : out_col + heads * dim] = out_scale * result."""
+    T = proj.shape[0]
+    H, D = heads, dim
+    HD = H * D
+    pf = proj.float()
+    rr = pf[:, r_off:r_off + HD].view(T, H, D)
+    k = pf[:, k_off:k_off + HD].view(T, H, D)
+    v = pf[:, v_off:v_off + HD].view(T, H, D)
+    g = pf[:, g_off:g_off + HD]
+    z = torch.tanh(pf[:, w_off:w_off + w_rank]) @ w2.float().T + w0.float()
+    w = torch.exp(-math.exp(-0.5) * torch.sigmoid(z)).view(T, H, D)
+    al = torch.sigmoid(pf[:, a_off:a_off + HD] + a_bias.float()).view(T, H, D)
+    u = k * torch.rsqrt((k * k).sum(-1, keepdim=True) + 1e-6)
+    o = torch.empty(T, H, D, dtype=torch.float32, device=proj.device)
+    for r, a, b, start, slot in _spans(batch):
+        S = state[slot].clone()
+        for t in range(a, b):
+            uS = torch.einsum("hd,hde->he", u[t], S)
+            S = w[t][:, :, None] * S - (al[t] * u[t])[:, :, None] * uS[:, None, :] + k[t][:, :, None] * v[t][:, None, :]
+            o[t] = torch.einsum("hde,hd->he", S, rr[t])
+        state[slot] = S
+    o = o * torch.rsqrt((o * o).mean(-1, keepdim=True) + eps)
+    o = o.reshape(T, HD) * norm_w.float() * torch.sigmoid(g)
+    out[:, out_col:out_col + HD] = (o * out_scale).to(out.dtype)
+
+
+def moe_route(logits, experts, top, groups, keep, scale):
+    """Sigmoid scores of the first ``experts`` logit columns; the ``top`` largest
+    are chosen, among the experts of the best ``keep`` of ``groups`` neighbour
+    groups when groups > 1 (a group's score: sum of its two largest scores);
+    weights = chosen scores / (their sum + 1e-20) * scale.
+    -> (ids [T, top] int32, weights [T, top] fp32)."""
+    from megatron_amd.moe.router import group_limited_topk
+
+    s = torch.sigmoid(logits[:, :experts].float())
+    if groups > 1:
+        _, idx = group_limited_topk(s, top, groups, keep)
+    else:
+        idx = s.topk(top, dim=-1).indices
+    sc = s.gather(1, idx)
+    return idx.to(torch.int32), sc / (sc.sum(-1, keepdim=True) + 1e-20) * scale
+
+
+def clamped_glu(gu, limit, alpha, out_dtype):
+    """gu [N, 2F] = [gate | up]: g = min(gate, limit), u = clamp(up, -limit, limit),
+    y = g sigmoid(alpha g) (u + 1)."""
+    F_ = gu.shape[1] // 2
+    g = torch.clamp(gu[:, :F_].float(), max=limit)
+    u = torch.clamp(gu[:, F_:].float(), -limit, limit)
+    return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(out_dtype)
+
+
+def moe_combine(down, inv, weights, shared, shared_gate, add):
+    """y[t] = sum_k weights[t, k] down[inv[t, k]] (+ sigmoid(shared_gate[t]) shared[t]) (+ add[t]), fp32."""
+    T, K = weights.shape
+    y = (down.float()[inv.long().view(-1)].view(T, K, -1) * weights[:, :, None]).sum(1)
+    if shared is not None:
+        y = y + torch.sigmoid(shared_gate.float())[:, None] * shared.float()
+    if add is not None:
+        y = y + add.float()
+    return y
