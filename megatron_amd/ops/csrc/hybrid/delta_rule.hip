@@ -1,0 +1,173 @@
+// Generalized delta rule over ragged batches with a per-request fp32 state:
+//   S <- diag(w) S - (a u)(u^T S) + k v^T ,  o = S^T r      (per head; both terms read the old S)
+//   w = exp(-e^{-1/2} sigmoid(W2 tanh(b) + w0)),  a = sigmoid(a_pre + a_b),  u = k / sqrt(sum k^2 + 1e-6)
+// The update is independent per value column: S[:, c] needs u . S[:, c] and
+// r . S[:, c] only.  Workgroup = (request, head, tile of 64 value columns);
+// thread (c, rg) holds rows rg * RPT .. rg * RPT + RPT - 1 of column c in
+// registers (RG = 1: a whole column, no cross-thread traffic in the token
+// loop).  A request's new tokens are walked in order; operands are staged in
+// LDS a chunk of tokens at a time, where all the non-linearities are
+// evaluated in parallel.
+#include "../ragged/ragged_common.h"
+
+constexpr int DR_COLS = 64;          // value columns per workgroup (one wave per row group)
+constexpr int DR_MAX_RANK = 128;     // decay bottleneck
+
+template <typename T, int DMAX, int RG, int CH>
+__global__ __launch_bounds__(DR_COLS * RG) void delta_rule_kernel(
+    const T* __restrict__ proj, long stride, int r_off, int k_off, int v_off, int a_off, int w_off, int rank,
+    const float* __restrict__ w2, const float* __restrict__ w0, const float* __restrict__ a_b,
+    float* __restrict__ state, const int* __restrict__ cu, const int* __restrict__ slots, float* __restrict__ o,
+    int H, int D) {
+  constexpr int RPT = DMAX / RG;
+  constexpr int NT = DR_COLS * RG;
+  __shared__ float s_r[CH][DMAX], s_k[CH][DMAX], s_u[CH][DMAX], s_au[CH][DMAX], s_w[CH][DMAX];
+  __shared__ float s_v[CH][DR_COLS], s_b[CH][DR_MAX_RANK], s_inv[CH];
+  __shared__ float red1[2][RG][DR_COLS], red2[2][RG][DR_COLS];
+  const int r = blockIdx.x, hd = blockIdx.y, ct = blockIdx.z;
+  const int c = threadIdx.x % DR_COLS, rg = threadIdx.x / DR_COLS;     // a wave = one row group
+  const int col = ct * DR_COLS + c;
+  const bool colok = col < D;
+  const long slot = slots[r];
+  float* sp = state + ((slot * H + hd) * D) * (long)D;
+  float S[RPT];
+#pragma unroll
+  for (int i = 0; i < RPT; ++i) {
+    const int row = rg * RPT + i;
+    S[i] = (row < D && colok) ? sp[(long)row * D + col] : 0.f;
+  }
+  const int t0 = cu[r], t1 = cu[r + 1];
+  const float decay_c = -0.60653065971263342f;     // -e^{-1/2}
+  int step = 0;
+  for (int tc = t0; tc < t1; tc += CH) {
+    const int nc = min(CH, t1 - tc);
+    for (int i = threadIdx.x; i < nc * rank; i += NT) {
+      const int tt = i / rank, j = i % rank;
+      s_b[tt][j] = tanhf(ldf(proj + (long)(tc + tt) * stride + w_off + j));
+    }
+    for (int i = threadIdx.x; i < nc * DR_COLS; i += NT) {
+      const int tt = i / DR_COLS, cc = ct * DR_COLS + i % DR_COLS;
+      s_v[tt][i % DR_COLS] = (cc < D) ? ldf(proj + (long)(tc + tt) * stride + v_off + hd * D + cc) : 0.f;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < nc * D; i += NT) {
+      const int tt = i / D, d = i % D, ch = hd * D + d;
+      const T* row = proj + (long)(tc + tt) * stride;
+      s_r[tt][d] = ldf(row + r_off + ch);
+      s_k[tt][d] = ldf(row + k_off + ch);
+      float z = w0[ch];
+      const float* w2r = w2 + (long)ch * rank;
+      for (int j = 0; j < rank; ++j) z += w2r[j] * s_b[tt][j];
+      s_w[tt][d] = expf(decay_c * sigmoidf_(z));
+      s_au[tt][d] = sigmoidf_(ldf(row + a_off + ch) + a_b[ch]);          // a for now, a * u below
+    }
+    __syncthreads();
+    for (int tt = rg; tt < nc; tt += RG) {          // one wave per token: squared norm of the key
+      float ss = 0.f;
+      for (int d = c; d < D; d += DR_COLS) ss += s_k[tt][d] * s_k[tt][d];
+      ss = wave_reduce_sum(ss);
+      if (c == 0) s_inv[tt] = 1.f / sqrtf(ss + 1e-6f);
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < nc * D; i += NT) {
+      const int tt = i / D, d = i % D;
+      const float u = s_k[tt][d] * s_inv[tt];
+      s_u[tt][d] = u;
+      s_au[tt][d] *= u;
+    }
+    __syncthreads();
+    for (int tt = 0; tt < nc; ++tt, ++step) {
+      const float vv = s_v[tt][c];
+      float dot = 0.f;
+#pragma unroll
+      for (int i = 0; i < RPT; ++i) dot += s_u[tt][rg * RPT + i] * S[i];     // rows >= D hold zeros in S
+      if constexpr (RG > 1) {
+        red1[step & 1][rg][c] = dot;
+        __syncthreads();
+        dot = 0.f;
+#pragma unroll
+        for (int g = 0; g < RG; ++g) dot += red1[step & 1][g][c];
+      }
+      float part = 0.f;
+#pragma unroll
+      for (int i = 0; i < RPT; ++i) {
+        const int row = rg * RPT + i;
+        if (row < D) {
+          S[i] = s_w[tt][row] * S[i] - s_au[tt][row] * dot + s_k[tt][row] * vv;
+          part += s_r[tt][row] * S[i];
+        }
+      }
+      if constexpr (RG > 1) {
+        red2[step & 1][rg][c] = part;
+        __syncthreads();
+        part = 0.f;
+#pragma unroll
+        for (int g = 0; g < RG; ++g) part += red2[step & 1][g][c];
+      }
+      if (rg == 0 && colok) o[((long)(tc + tt) * H + hd) * D + col] = part;
+    }
+    __syncthreads();                                // the chunk buffers are rewritten next
+  }
+#pragma unroll
+  for (int i = 0; i < RPT; ++i) {
+    const int row = rg * RPT + i;
+    if (row < D && colok) sp[(long)row * D + col] = S[i];
+  }
+}
+
+// per-head RMS norm of o, learned weight, sigmoid output gate, output scale; one wave per (token, head)
+template <typename T>
+__global__ __launch_bounds__(256) void delta_out_kernel(const float* __restrict__ o, const T* __restrict__ proj,
+                                                        long stride, int g_off, const float* __restrict__ w,
+                                                        float eps, T* __restrict__ out, long out_stride, int out_col,
+                                                        float out_scale, int TH, int H, int D) {
+  const int wid = blockIdx.x * (256 / WAVE) + threadIdx.x / WAVE;
+  const int lane = threadIdx.x % WAVE;
+  if (wid >= TH) return;
+  const int t = wid / H, hd = wid % H;
+  const float* op = o + (long)wid * D;
+  float ss = 0.f;
+  for (int d = lane; d < D; d += WAVE) ss += op[d] * op[d];
+  const float rs = 1.f / sqrtf(wave_reduce_sum(ss) / (float)D + eps);
+  const T* gp = proj + (long)t * stride + g_off + (long)hd * D;
+  T* dst = out + (long)t * out_stride + out_col + (long)hd * D;
+  for (int d = lane; d < D; d += WAVE)
+    stf(dst + d, op[d] * rs * w[hd * D + d] * sigmoidf_(ldf(gp + d)) * out_scale);
+}
+
+void delta_rule_scan(torch::Tensor proj, int64_t r_off, int64_t k_off, int64_t v_off, int64_t g_off, int64_t a_off,
+                     int64_t w_off, int64_t rank, torch::Tensor w2, torch::Tensor w0, torch::Tensor a_b,
+                     torch::Tensor norm_w, int64_t H, int64_t D, double eps, torch::Tensor state, torch::Tensor cu,
+                     torch::Tensor slots, torch::Tensor out, int64_t out_col, double out_scale) {
+  TORCH_CHECK(proj.is_cuda() && proj.dim() == 2 && proj.stride(1) == 1);
+  check_f32(w2, "w2"); check_f32(w0, "w0"); check_f32(a_b, "a bias"); check_f32(norm_w, "norm"); check_f32(state, "S");
+  check_i32(cu, "cu"); check_i32(slots, "slots");
+  const int T_ = proj.size(0), C = proj.size(1), R = slots.numel();
+  const long HD = H * D;
+  for (int64_t off : {r_off, k_off, v_off, g_off, a_off}) TORCH_CHECK(off >= 0 && off + HD <= C, "column slice");
+  TORCH_CHECK(w_off >= 0 && w_off + rank <= C && rank >= 1 && rank <= DR_MAX_RANK, "decay bottleneck above ", DR_MAX_RANK);
+  TORCH_CHECK(w2.numel() == HD * rank && w0.numel() == HD && a_b.numel() == HD && norm_w.numel() == HD);
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == D && state.size(3) == D && cu.numel() == R + 1);
+  TORCH_CHECK(D <= 256, "delta-rule head dim above 256");
+  TORCH_CHECK(out.is_cuda() && out.dim() == 2 && out.stride(1) == 1 && out.size(0) == T_ &&
+              out.scalar_type() == proj.scalar_type() && out_col >= 0 && out_col + HD <= out.size(1));
+  if (T_ == 0 || R == 0) return;
+  auto o = torch::empty({T_, H, D}, proj.options().dtype(at::kFloat));
+  auto stream = at::cuda::getCurrentHIPStream();
+  const dim3 grid(R, (unsigned)H, (unsigned)((D + DR_COLS - 1) / DR_COLS));
+#define DR_LAUNCH(DMAX, RG, CH)                                                                                \
+  hipLaunchKernelGGL((delta_rule_kernel<T, DMAX, RG, CH>), grid, dim3(DR_COLS * RG), 0, stream,                \
+      (const T*)proj.data_ptr(), (long)proj.stride(0), (int)r_off, (int)k_off, (int)v_off, (int)a_off,         \
+      (int)w_off, (int)rank, w2.data_ptr<float>(), w0.data_ptr<float>(), a_b.data_ptr<float>(),                \
+      state.data_ptr<float>(), cu.data_ptr<int>(), slots.data_ptr<int>(), o.data_ptr<float>(), (int)H, (int)D)
+  RAGGED_DISPATCH(proj, {
+    if (D <= 64) DR_LAUNCH(64, 1, 16);
+    else if (D <= 128) DR_LAUNCH(128, 2, 16);
+    else DR_LAUNCH(256, 4, 8);
+    const int TH = T_ * H;
+    hipLaunchKernelGGL((delta_out_kernel<T>), dim3((TH + 3) / 4), dim3(256), 0, stream, o.data_ptr<float>(),
+        (const T*)proj.data_ptr(), (long)proj.stride(0), (int)g_off, norm_w.data_ptr<float>(), (float)eps,
+        (T*)out.data_ptr(), (long)out.stride(0), (int)out_col, (float)out_scale, TH, (int)H, (int)D);
+  });
+#undef DR_LAUNCH
+}

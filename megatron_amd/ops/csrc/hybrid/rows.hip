@@ -1,0 +1,249 @@
+// Row kernels of the plain-residual serving path: embedding gather into the
+// fp32 residual, residual add fused with grouped RMS norm (one or two normed
+// copies of the same row), and the elementwise / per-token parts of routed
+// clamped-GLU experts (routing, activation, weighted combine).
+#include "../ragged/ragged_common.h"
+
+// ---------------------------------------------------------------------------
+// x[t] = embed[token[t]]  (fp32)
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void embed_plain_kernel(const long* __restrict__ tokens, const T* __restrict__ embed,
+                                   float* __restrict__ x, int W) {
+  const long t = blockIdx.x;
+  const T* row = embed + tokens[t] * (long)W;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) x[t * W + c] = ldf(row + c);
+}
+
+torch::Tensor embed_plain(torch::Tensor tokens, torch::Tensor embed) {
+  TORCH_CHECK(tokens.is_cuda() && tokens.scalar_type() == at::kLong && tokens.is_contiguous() && tokens.dim() == 1);
+  TORCH_CHECK(embed.is_cuda() && embed.dim() == 2 && embed.is_contiguous());
+  const int T_ = tokens.numel(), W = embed.size(1);
+  auto x = torch::empty({T_, W}, embed.options().dtype(at::kFloat));
+  if (T_ == 0) return x;
+  auto stream = at::cuda::getCurrentHIPStream();
+  RAGGED_DISPATCH(embed, hipLaunchKernelGGL((embed_plain_kernel<T>), dim3(T_), dim3(256), 0, stream,
+      tokens.data_ptr<long>(), (const T*)embed.data_ptr(), x.data_ptr<float>(), W));
+  return x;
+}
+
+// ---------------------------------------------------------------------------
+// x += y ; n = x / rms(x) per group ; h_a = n * w_a ; h_b = n * w_b
+// One workgroup per token; the row is staged in LDS, wave w reduces the
+// groups w, w + 4, ...
+// ---------------------------------------------------------------------------
+constexpr int GN_MAX_GROUPS = 256;
+
+template <typename TY, typename TO>
+__global__ __launch_bounds__(256) void residual_group_norm_kernel(
+    float* __restrict__ x, const TY* __restrict__ y, const float* __restrict__ wa, const float* __restrict__ wb,
+    TO* __restrict__ ha, TO* __restrict__ hb, int W, int groups, float eps) {
+  extern __shared__ float row[];
+  __shared__ float rs[GN_MAX_GROUPS];
+  const long t = blockIdx.x;
+  float* xp = x + t * W;
+  for (int c = threadIdx.x; c < W; c += 256) {
+    float v = xp[c];
+    if (y != nullptr) {
+      v += ldf(y + t * W + c);
+      xp[c] = v;
+    }
+    row[c] = v;
+  }
+  __syncthreads();
+  const int gs = W / groups, wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  for (int g = wave; g < groups; g += 4) {
+    float ss = 0.f;
+    for (int i = lane; i < gs; i += WAVE) {
+      const float v = row[g * gs + i];
+      ss += v * v;
+    }
+    ss = wave_reduce_sum(ss);
+    if (lane == 0) rs[g] = 1.f / sqrtf(ss / (float)gs + eps);
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < W; c += 256) {
+    const float n = row[c] * rs[c / gs];
+    stf(ha + t * W + c, n * wa[c]);
+    if (hb != nullptr) stf(hb + t * W + c, n * wb[c]);
+  }
+}
+
+std::vector<torch::Tensor> residual_group_norm(torch::Tensor x, torch::Tensor y, torch::Tensor wa, torch::Tensor wb,
+                                               int64_t groups, double eps, bool out_bf16) {
+  check_f32(x, "x"); check_f32(wa, "w_a");
+  TORCH_CHECK(x.dim() == 2);
+  const int T_ = x.size(0), W = x.size(1);
+  const bool has_y = y.numel() > 0, has_b = wb.numel() > 0;
+  TORCH_CHECK(groups >= 1 && groups <= GN_MAX_GROUPS && W % groups == 0, "norm groups divide the width");
+  TORCH_CHECK(wa.numel() == W && (!has_b || (wb.numel() == W && wb.scalar_type() == at::kFloat && wb.is_cuda())));
+  if (has_y) {
+    TORCH_CHECK(y.is_cuda() && y.is_contiguous() && y.dim() == 2 && y.size(0) == T_ && y.size(1) == W);
+    TORCH_CHECK(y.scalar_type() == at::kFloat || y.scalar_type() == at::kBFloat16);
+  }
+  auto ho = x.options().dtype(out_bf16 ? at::kBFloat16 : at::kFloat);
+  auto ha = torch::empty({T_, W}, ho);
+  auto hb = has_b ? torch::empty({T_, W}, ho) : torch::empty({0}, ho);
+  if (T_ == 0) return {ha, hb};
+  auto stream = at::cuda::getCurrentHIPStream();
+  const size_t smem = (size_t)W * sizeof(float);
+  TORCH_CHECK(smem <= 96 * 1024, "row too wide for the norm kernel");
+#define GN_LAUNCH(TY, TO)                                                                                        \
+  hipLaunchKernelGGL((residual_group_norm_kernel<TY, TO>), dim3(T_), dim3(256), smem, stream, x.data_ptr<float>(), \
+      has_y ? (const TY*)y.data_ptr() : (const TY*)nullptr, wa.data_ptr<float>(),                                \
+      has_b ? wb.data_ptr<float>() : (const float*)nullptr, (TO*)ha.data_ptr(),                                  \
+      has_b ? (TO*)hb.data_ptr() : (TO*)nullptr, W, (int)groups, (float)eps)
+  const bool y_bf = has_y && y.scalar_type() == at::kBFloat16;
+  if (y_bf && out_bf16) GN_LAUNCH(bf16, bf16);
+  else if (y_bf) GN_LAUNCH(bf16, float);
+  else if (out_bf16) GN_LAUNCH(float, bf16);
+  else GN_LAUNCH(float, float);
+#undef GN_LAUNCH
+  return {ha, hb};
+}
+
+// ---------------------------------------------------------------------------
+// routing: sigmoid scores, group-limited top-k, normalised weights.
+// One thread per token.
+// ---------------------------------------------------------------------------
+constexpr int RT_MAX_TOP = 16, RT_MAX_GROUPS = 64;
+
+__global__ void moe_route_kernel(const float* __restrict__ logits, long stride, int Tn, int E, int top, int groups,
+                                 int keep, float scale, int* __restrict__ ids, float* __restrict__ wts) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= Tn) return;
+  const float* z = logits + (long)t * stride;
+  unsigned long long allowed = ~0ull;             // bit g: group g may be chosen from
+  const int per = E / groups;
+  if (groups > 1) {
+    float gsc[RT_MAX_GROUPS];
+    for (int g = 0; g < groups; ++g) {
+      float a = -1.f, b = -1.f;                   // two largest scores of the group (scores lie in (0, 1))
+      for (int i = 0; i < per; ++i) {
+        const float s = sigmoidf_(z[g * per + i]);
+        if (s > a) { b = a; a = s; }
+        else if (s > b) b = s;
+      }
+      gsc[g] = a + (per > 1 ? b : 0.f);
+    }
+    allowed = 0ull;
+    for (int n = 0; n < keep; ++n) {
+      int best = -1;
+      float bv = -INFINITY;
+      for (int g = 0; g < groups; ++g)
+        if (!((allowed >> g) & 1ull) && gsc[g] > bv) { bv = gsc[g]; best = g; }
+      if (best >= 0) allowed |= 1ull << best;
+    }
+  }
+  int chosen[RT_MAX_TOP];
+  float cs[RT_MAX_TOP];
+  float sum = 0.f;
+  for (int n = 0; n < top; ++n) {
+    int best = -1;
+    float bv = -INFINITY;
+    for (int e = 0; e < E; ++e) {
+      if (groups > 1 && !((allowed >> (e / per)) & 1ull)) continue;
+      bool taken = false;
+      for (int m = 0; m < n; ++m) taken |= chosen[m] == e;
+      if (taken) continue;
+      const float s = sigmoidf_(z[e]);
+      if (s > bv) { bv = s; best = e; }
+    }
+    chosen[n] = best < 0 ? 0 : best;
+    cs[n] = best < 0 ? 0.f : bv;
+    sum += cs[n];
+  }
+  for (int n = 0; n < top; ++n) {
+    ids[(long)t * top + n] = chosen[n];
+    wts[(long)t * top + n] = cs[n] / (sum + 1e-20f) * scale;
+  }
+}
+
+std::vector<torch::Tensor> moe_route(torch::Tensor logits, int64_t E, int64_t top, int64_t groups, int64_t keep,
+                                     double scale) {
+  TORCH_CHECK(logits.is_cuda() && logits.scalar_type() == at::kFloat && logits.dim() == 2 && logits.stride(1) == 1);
+  TORCH_CHECK(E >= 1 && E <= logits.size(1) && top >= 1 && top <= RT_MAX_TOP && top <= E, "experts chosen per token");
+  TORCH_CHECK(groups >= 1 && groups <= RT_MAX_GROUPS && E % groups == 0 && keep >= 1 && keep <= groups);
+  TORCH_CHECK(groups == 1 || keep * (E / groups) >= top, "the kept groups hold fewer experts than are chosen");
+  const int T_ = logits.size(0);
+  auto ids = torch::empty({T_, top}, logits.options().dtype(at::kInt));
+  auto wts = torch::empty({T_, top}, logits.options());
+  if (T_ == 0) return {ids, wts};
+  auto stream = at::cuda::getCurrentHIPStream();
+  hipLaunchKernelGGL(moe_route_kernel, dim3((T_ + 63) / 64), dim3(64), 0, stream, logits.data_ptr<float>(),
+                     (long)logits.stride(0), T_, (int)E, (int)top, (int)groups, (int)keep, (float)scale,
+                     ids.data_ptr<int>(), wts.data_ptr<float>());
+  return {ids, wts};
+}
+
+// ---------------------------------------------------------------------------
+// y = g sigmoid(alpha g) (u + 1),  g = min(gate, limit), u = clamp(up, -limit, limit)
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void clamped_glu_kernel(const T* __restrict__ gu, long stride, T* __restrict__ y, long N, int F,
+                                   float limit, float alpha) {
+  const long total = N * F;
+  for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+    const long n = i / F;
+    const int f = (int)(i % F);
+    const float g = fminf(ldf(gu + n * stride + f), limit);
+    const float u = fminf(fmaxf(ldf(gu + n * stride + F + f), -limit), limit);
+    stf(y + i, g * sigmoidf_(alpha * g) * (u + 1.f));
+  }
+}
+
+torch::Tensor clamped_glu(torch::Tensor gu, double limit, double alpha) {
+  TORCH_CHECK(gu.is_cuda() && gu.dim() == 2 && gu.stride(1) == 1 && gu.size(1) % 2 == 0);
+  const long N = gu.size(0);
+  const int F = gu.size(1) / 2;
+  auto y = torch::empty({N, F}, gu.options());
+  if (N == 0) return y;
+  auto stream = at::cuda::getCurrentHIPStream();
+  RAGGED_DISPATCH(gu, hipLaunchKernelGGL((clamped_glu_kernel<T>), dim3(grid_for(N * F, 256)), dim3(256), 0, stream,
+      (const T*)gu.data_ptr(), (long)gu.stride(0), (T*)y.data_ptr(), N, F, (float)limit, (float)alpha));
+  return y;
+}
+
+// ---------------------------------------------------------------------------
+// y[t] = sum_k w[t,k] down[inv[t,k]] + sigmoid(gate[t]) shared[t] + add[t]   (fp32)
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void moe_combine_kernel(
+    const T* __restrict__ down, const int* __restrict__ inv, const float* __restrict__ wts,
+    const T* __restrict__ shared, const float* __restrict__ gate, const T* __restrict__ add,
+    float* __restrict__ y, int W, int K) {
+  const long t = blockIdx.x;
+  const float sg = shared != nullptr ? sigmoidf_(gate[t]) : 0.f;
+  for (int c = threadIdx.x; c < W; c += 256) {
+    float a = 0.f;
+    for (int k = 0; k < K; ++k) a += wts[t * K + k] * ldf(down + (long)inv[t * K + k] * W + c);
+    if (shared != nullptr) a += sg * ldf(shared + t * W + c);
+    if (add != nullptr) a += ldf(add + t * W + c);
+    y[t * W + c] = a;
+  }
+}
+
+torch::Tensor moe_combine(torch::Tensor down, torch::Tensor inv, torch::Tensor wts, torch::Tensor shared,
+                          torch::Tensor gate, torch::Tensor add) {
+  TORCH_CHECK(down.is_cuda() && down.dim() == 2 && down.is_contiguous());
+  check_i32(inv, "inv"); check_f32(wts, "weights");
+  TORCH_CHECK(wts.dim() == 2 && inv.sizes() == wts.sizes());
+  const int T_ = wts.size(0), K = wts.size(1), W = down.size(1);
+  TORCH_CHECK(down.size(0) == (long)T_ * K);
+  const bool has_s = shared.numel() > 0, has_a = add.numel() > 0;
+  if (has_s) {
+    TORCH_CHECK(shared.is_contiguous() && shared.scalar_type() == down.scalar_type() && shared.size(0) == T_ &&
+                shared.size(1) == W);
+    check_f32(gate, "shared gate");
+    TORCH_CHECK(gate.numel() == T_);
+  }
+  if (has_a) TORCH_CHECK(add.is_contiguous() && add.scalar_type() == down.scalar_type() && add.size(0) == T_ && add.size(1) == W);
+  auto y = torch::empty({T_, W}, down.options().dtype(at::kFloat));
+  if (T_ == 0) return y;
+  auto stream = at::cuda::getCurrentHIPStream();
+  RAGGED_DISPATCH(down, hipLaunchKernelGGL((moe_combine_kernel<T>), dim3(T_), dim3(256), 0, stream,
+      (const T*)down.data_ptr(), inv.data_ptr<int>(), wts.data_ptr<float>(),
+      has_s ? (const T*)shared.data_ptr() : (const T*)nullptr, has_s ? gate.data_ptr<float>() : (const float*)nullptr,
+      has_a ? (const T*)add.data_ptr() : (const T*)nullptr, y.data_ptr<float>(), W, K));
+  return y;
+}

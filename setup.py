@@ -40,8 +40,16 @@ RAGGED_SRC = [
     "megatron_amd/ops/csrc/ragged/latent_attention_mfma.hip",
 ]
 
+HYBRID_SRC = [
+    "megatron_amd/ops/csrc/hybrid/bindings.cpp",
+    "megatron_amd/ops/csrc/hybrid/rows.hip",
+    "megatron_amd/ops/csrc/hybrid/window_attention.hip",
+    "megatron_amd/ops/csrc/hybrid/delta_rule.hip",
+]
+
 # MEGATRON_AMD_ONLY_EXT=ragged builds just the serving kernels of the
-# ragged-batch models (what a fresh checkout compiles on first use)
+# ragged-batch models (what a fresh checkout compiles on first use); "hybrid"
+# likewise for the models built on the hybrid kernels
 ONLY = os.environ.get("MEGATRON_AMD_ONLY_EXT", "")
 
 EXTS = {
@@ -59,6 +67,12 @@ EXTS = {
         CUDAExtension(
             name="megatron_amd.ops._ragged_ops",
             sources=RAGGED_SRC,
+            extra_compile_args={"cxx": ["-O3", "-std=c++17"], "nvcc": HIPCC_FLAGS},
+        ),
+    "hybrid": lambda:
+        CUDAExtension(
+            name="megatron_amd.ops._hybrid_ops",
+            sources=HYBRID_SRC,
             extra_compile_args={"cxx": ["-O3", "-std=c++17"], "nvcc": HIPCC_FLAGS},
         ),
     "data": lambda:
