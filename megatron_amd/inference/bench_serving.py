@@ -1,4 +1,4 @@
-"""Serving throughput of ragged-batch models beside the closest dense model.
+"""Serving throughput of ragged-batch models beside the closest existing model.
 
 For each size: random-init weights, bf16, synthetic prompts.  Prefill =
 ``batch`` prompts of ``isl`` tokens run to their last token; decode = ``osl``
@@ -8,6 +8,11 @@ comparison model is GPTModel with multi-latent attention at the same width,
 depth, heads and ranks through the same engine class (its paged-latent path:
 one prompt per prefill step, batched decode steps).  One JSON line per
 (size, model), tokens/s for both phases.
+
+``--serve-design bezurax`` measures the Bezurax design (pooled-window attention
+beside a delta-rule memory, routed experts) next to the Bezutar design with
+alternating attention / mLSTM layers at the same width, depth and active
+feed-forward size, both through the same ragged engine path.
 """
 
 from __future__ import annotations
@@ -45,6 +50,31 @@ def bezutar_config(s, pattern, max_pos):
                 embedding=dict(bigram=dict(buckets=50021, mul_prev=31, mul_cur=17)), layers=layers)
 
 
+# Bezurax at the same widths and depths: query heads x 128, a quarter as many kv heads,
+# window 1024 with 16-token pooled blocks; delta-rule heads of 64; 16 experts of which 3
+# are chosen plus a shared one: the active feed-forward size equals the dense ff above
+X_SIZES = {
+    "1b": dict(heads=16, kv=4, dim=128, window=1024, pool=16, r_heads=16, r_dim=64, experts=16, top=3, eff=1408,
+               sff=1408, groups=4, keep=2),
+    "7b-layers": dict(heads=32, kv=8, dim=128, window=1024, pool=16, r_heads=32, r_dim=64, experts=16, top=3,
+                      eff=2752, sff=2752, groups=4, keep=2),
+}
+
+
+def bezurax_config(size):
+    s, x = SIZES[size], X_SIZES[size]
+    one = dict(type="parallel",
+               mixer=dict(left=dict(heads=x["heads"], kv_heads=x["kv"], dim=x["dim"], vdim=x["dim"],
+                                    scale=x["dim"] ** -0.5, mask=dict(size=x["window"], pool=x["pool"])),
+                          right=dict(heads=x["r_heads"], dim=x["r_dim"]), left_scale=1.0, right_scale=1.0),
+               mlp=dict(kind="moe", expert=dict(ff=x["eff"], limit=7.0),
+                        router=dict(experts=x["experts"], top=x["top"], scale=1.0,
+                                    groups=dict(count=x["groups"], keep=x["keep"])),
+                        shared=dict(ff=x["sff"], limit=7.0)))
+    return dict(architecture="Bezurax", vocab=s["vocab"], width=s["width"], norm=dict(eps=1e-6, groups=4),
+                logit_scale=1.0, layers=[json.loads(json.dumps(one)) for _ in range(s["layers"])])
+
+
 def _random_init(model, seed=0):
     g = torch.Generator(device="cpu").manual_seed(seed)
     with torch.no_grad():
@@ -52,7 +82,7 @@ def _random_init(model, seed=0):
             if p.dim() >= 2 and p.dtype != torch.float32:
                 fan_in = p.shape[-1]
                 p.copy_((torch.randn(p.shape, generator=g) * fan_in ** -0.5).to(p.dtype))
-            elif name.endswith("w_gates"):
+            elif name.endswith(("w_gates", "w_router", "w2")):
                 p.copy_(torch.randn(p.shape, generator=g) * p.shape[-1] ** -0.5)
             elif name.endswith("weight") and p.dim() == 2:      # canon taps
                 p.copy_(torch.randn(p.shape, generator=g) * 0.2)
@@ -68,7 +98,6 @@ def _time(fn):
 
 
 def run_bezutar(size, pattern, batch, isl, osl, device):
-    from megatron_amd.inference.engine import DynamicInferenceEngine
     from megatron_amd.models.bezutar import BezutarConfig, BezutarModel
 
     s = SIZES[size]
@@ -76,6 +105,23 @@ def run_bezutar(size, pattern, batch, isl, osl, device):
     with torch.device(device):
         model = BezutarModel(cfg).eval()
     _random_init(model)
+    return _run_ragged(model, f"bezutar[{pattern}]", size, batch, isl, osl, device)
+
+
+def run_bezurax(size, batch, isl, osl, device):
+    from megatron_amd.models.bezurax import BezuraxConfig, BezuraxModel
+
+    cfg = BezuraxConfig.from_dict(bezurax_config(size), dtype=torch.bfloat16)
+    with torch.device(device):
+        model = BezuraxModel(cfg).eval()
+    _random_init(model)
+    return _run_ragged(model, "bezurax", size, batch, isl, osl, device)
+
+
+def _run_ragged(model, label, size, batch, isl, osl, device):
+    from megatron_amd.inference.engine import DynamicInferenceEngine
+
+    s = SIZES[size]
     page = 64
     eng = DynamicInferenceEngine(model, num_blocks=batch * ((isl + osl) // page + 2), block_size=page,
                                  max_batch=batch, device=device, use_hip_graphs=False,
@@ -99,7 +145,7 @@ def run_bezutar(size, pattern, batch, isl, osl, device):
     once()                      # warm-up (GEMM algorithm selection, allocator)
     t_pre, t_dec = once()
     n = sum(p.numel() for p in model.parameters())
-    return dict(model=f"bezutar[{pattern}]", size=size, params_m=round(n / 1e6, 1),
+    return dict(model=label, size=size, params_m=round(n / 1e6, 1),
                 prefill_tok_s=round(batch * isl / t_pre, 1), decode_tok_s=round(batch * osl / t_dec, 1),
                 prefill_ms=round(1e3 * t_pre, 2), decode_ms_per_step=round(1e3 * t_dec / osl, 3))
 
@@ -160,6 +206,11 @@ def main(args) -> None:
     device = torch.device("cuda", 0)
     torch.cuda.set_device(0)
     for size in args.serve_sizes.split(","):
+        if getattr(args, "serve_design", "bezutar") == "bezurax":
+            r = run_bezurax(size, args.serve_batch, args.serve_isl, args.serve_osl, device)
+            r.update(batch=args.serve_batch, isl=args.serve_isl, osl=args.serve_osl, dtype="bf16", data="synthetic")
+            print(json.dumps(r), flush=True)
+            torch.cuda.empty_cache()
         for pattern in [p for p in args.serve_patterns.split(",") if p and p != "none"]:
             r = run_bezutar(size, pattern, args.serve_batch, args.serve_isl, args.serve_osl, device)
             r.update(batch=args.serve_batch, isl=args.serve_isl, osl=args.serve_osl, dtype="bf16", data="synthetic")

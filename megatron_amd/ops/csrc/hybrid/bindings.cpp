@@ -21,6 +21,11 @@ void pooled_window_attention(torch::Tensor q, torch::Tensor pool, torch::Tensor 
                              int64_t D, int64_t V, double scale, int64_t window, int64_t P, int64_t rpp,
                              torch::Tensor tok_req, torch::Tensor tok_pos, torch::Tensor tables, int64_t bs,
                              torch::Tensor out, int64_t out_col, double out_scale);
+void pooled_window_attention_mfma(torch::Tensor q, torch::Tensor pool, torch::Tensor pooled, int64_t H, int64_t G,
+                                  int64_t D, int64_t V, double scale, int64_t window, int64_t P, int64_t rpp,
+                                  torch::Tensor tiles, torch::Tensor cu, torch::Tensor start_pos,
+                                  torch::Tensor tables, int64_t bs, int64_t nsplit, torch::Tensor out,
+                                  int64_t out_col, double out_scale);
 void delta_rule_scan(torch::Tensor proj, int64_t r_off, int64_t k_off, int64_t v_off, int64_t g_off, int64_t a_off,
                      int64_t w_off, int64_t rank, torch::Tensor w2, torch::Tensor w0, torch::Tensor a_b,
                      torch::Tensor norm_w, int64_t H, int64_t D, double eps, torch::Tensor state, torch::Tensor cu,
@@ -35,5 +40,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("qk_norm_store", &qk_norm_store);
   m.def("pool_blocks", &pool_blocks);
   m.def("pooled_window_attention", &pooled_window_attention);
+  m.def("pooled_window_attention_mfma", &pooled_window_attention_mfma);
   m.def("delta_rule_scan", &delta_rule_scan);
 }

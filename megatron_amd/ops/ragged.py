@@ -260,6 +260,19 @@ def pool_blocks(pool, pooled, block, pooled_per_page, batch):
 def pooled_window_attention(q, pool, pooled, heads, kv_heads, dim, vdim, scale, window, block,
                             pooled_per_page, batch, out, out_col, out_scale):
     if _native_h(q):
+        if (q.dtype == torch.bfloat16 and dim % 8 == 0 and vdim % 8 == 0 and dim <= 256 and vdim <= 256
+                and os.environ.get("MEGATRON_AMD_NO_MFMA_WINDOW", "0") != "1"):
+            # matrix-core kernel: 64 (token, head-in-group) rows per workgroup and kv head; steps
+            # with few rows (decode) also split the key tiles over workgroups
+            tiles = batch.row_tiles(heads // kv_heads, q.device)
+            nblk = tiles.shape[0] * kv_heads
+            keys = min(batch.max_context, window + 64 + batch.max_context // block)
+            nsplit = max(1, min((keys + 63) // 64, 1024 // max(nblk, 1), 64))
+            _H.pooled_window_attention_mfma(q, pool, pooled, int(heads), int(kv_heads), int(dim), int(vdim),
+                                            float(scale), int(window), int(block), int(pooled_per_page), tiles,
+                                            batch.cu_tokens, batch.start_pos, batch.block_tables,
+                                            int(batch.block_size), int(nsplit), out, int(out_col), float(out_scale))
+            return
         _H.pooled_window_attention(q, pool, pooled, int(heads), int(kv_heads), int(dim), int(vdim), float(scale),
                                    int(window), int(block), int(pooled_per_page), batch.tok_req, batch.tok_pos,
                                    batch.block_tables, int(batch.block_size), out, int(out_col), float(out_scale))

@@ -49,11 +49,15 @@ def test_embed_and_group_norm(dtype, groups):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("shape", [(4, 2, 24, 24, 9, 4), (3, 3, 80, 80, 5, 1), (6, 1, 136, 136, 64, 7), (2, 2, 16, 16, 1, 3)])
-def test_pooled_window_attention(dtype, shape):
-    """heads, kv heads, dim, vdim, window, pool; page 16: pooled rows and windows cross pages"""
+@pytest.mark.parametrize("shape", [(4, 2, 24, 24, 9, 4), (3, 3, 80, 80, 5, 1), (6, 1, 136, 136, 64, 7), (2, 2, 16, 16, 1, 3),
+                                   (8, 2, 64, 64, 40, 6)])
+@pytest.mark.parametrize("starts", [STARTS, [0, 300, 130, 3, 517]], ids=["short", "long"])
+def test_pooled_window_attention(dtype, shape, starts):
+    """heads, kv heads, dim, vdim, window, pool; page 16: pooled rows and windows cross pages;
+    long contexts beside short ones make the bf16 kernel split the key tiles over workgroups"""
     R = _need()
     H, G, D, V, window, P = shape
+    STARTS = starts
     bs = 16
     rpp = (bs + P - 1) // P
 
