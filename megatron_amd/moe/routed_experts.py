@@ -11,11 +11,13 @@ y = g sigmoid(alpha g) (u + 1), output W_down y.
 Optional shared expert of the same form for every token, times
 sigmoid(w_sg . h); its gate row rides in the fp32 router GEMM.
 
-Step: one fp32 GEMM [router; shared gate], a routing kernel, then the
-(token, choice) pairs are sorted by expert and each expert with work runs its
-gate/up and down products on its slice (vendor GEMMs; the pair counts are the
-step's one host read), and one kernel forms
-sum_k weight_k down_k + sigmoid(gate) shared + add in fp32.
+Step: one fp32 GEMM [router; shared gate], a routing kernel, then
+  * many pairs (prompt portions): the (token, choice) pairs are sorted by expert
+    and each expert with work runs its gate/up and down products on its slice
+    (vendor GEMMs; the pair counts are the step's one host read),
+  * few pairs (decoding): two kernels in which every pair streams its expert's
+    matrices (ops.ragged.expert_pairs), no sort and no host read,
+and one kernel forms sum_k weight_k down_k + sigmoid(gate) shared + add in fp32.
 """
 
 from __future__ import annotations
@@ -58,6 +60,16 @@ class RoutedExpertsMLP(nn.Module):
         """h [T, hidden] in the compute dtype -> fp32 [T, hidden] (+ add)."""
         T, K, E = h.shape[0], self.top, self.experts
         logits, ids, weights = self.route(h)
+        shared = gate = None
+        if self.shared_ff:
+            sy = R.clamped_glu(F.linear(h, self.ws_gate_up), self.shared_limit, self.alpha, h.dtype)
+            shared = F.linear(sy, self.ws_down)
+            gate = logits[:, E].contiguous()
+        if R.expert_pairs_ok(h, K, self.ff):
+            # few pairs (decoding): each pair streams its expert's matrices, no sort, no host read
+            down = R.expert_pairs(h, ids, self.w_gate_up, self.w_down, self.limit, self.alpha)
+            inv = torch.arange(T * K, dtype=torch.int32, device=h.device).view(T, K)
+            return R.moe_combine(down, inv, weights, shared, gate, add)
         flat = ids.reshape(-1).long()
         order = torch.argsort(flat, stable=True)              # pairs sorted by expert
         inv = torch.empty_like(order)
@@ -71,9 +83,4 @@ class RoutedExpertsMLP(nn.Module):
                 gu = F.linear(xs[at:at + n], self.w_gate_up[e])
                 down[at:at + n] = F.linear(R.clamped_glu(gu, self.limit, self.alpha, h.dtype), self.w_down[e])
                 at += n
-        shared = gate = None
-        if self.shared_ff:
-            sy = R.clamped_glu(F.linear(h, self.ws_gate_up), self.shared_limit, self.alpha, h.dtype)
-            shared = F.linear(sy, self.ws_down)
-            gate = logits[:, E].contiguous()
         return R.moe_combine(down, inv.view(T, K).to(torch.int32), weights, shared, gate, add)

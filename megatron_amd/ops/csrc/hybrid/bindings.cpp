@@ -12,6 +12,8 @@ std::vector<torch::Tensor> moe_route(torch::Tensor logits, int64_t E, int64_t to
 torch::Tensor clamped_glu(torch::Tensor gu, double limit, double alpha);
 torch::Tensor moe_combine(torch::Tensor down, torch::Tensor inv, torch::Tensor wts, torch::Tensor shared,
                           torch::Tensor gate, torch::Tensor add);
+torch::Tensor expert_pairs(torch::Tensor h, torch::Tensor ids, torch::Tensor wgu, torch::Tensor wd, double limit,
+                           double alpha);
 torch::Tensor qk_norm_store(torch::Tensor proj, int64_t q_off, int64_t qw, int64_t k_off, int64_t kw, int64_t v_off,
                             int64_t vw, torch::Tensor wq, torch::Tensor wk, double eps, torch::Tensor pool,
                             torch::Tensor tok_row);
@@ -37,6 +39,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("moe_route", &moe_route);
   m.def("clamped_glu", &clamped_glu);
   m.def("moe_combine", &moe_combine);
+  m.def("expert_pairs", &expert_pairs);
   m.def("qk_norm_store", &qk_norm_store);
   m.def("pool_blocks", &pool_blocks);
   m.def("pooled_window_attention", &pooled_window_attention);

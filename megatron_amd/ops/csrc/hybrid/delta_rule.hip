@@ -2,30 +2,35 @@
 //   S <- diag(w) S - (a u)(u^T S) + k v^T ,  o = S^T r      (per head; both terms read the old S)
 //   w = exp(-e^{-1/2} sigmoid(W2 tanh(b) + w0)),  a = sigmoid(a_pre + a_b),  u = k / sqrt(sum k^2 + 1e-6)
 // The update is independent per value column: S[:, c] needs u . S[:, c] and
-// r . S[:, c] only.  Workgroup = (request, head, tile of 64 value columns);
-// thread (c, rg) holds rows rg * RPT .. rg * RPT + RPT - 1 of column c in
-// registers (RG = 1: a whole column, no cross-thread traffic in the token
-// loop).  A request's new tokens are walked in order; operands are staged in
-// LDS a chunk of tokens at a time, where all the non-linearities are
-// evaluated in parallel.
+// r . S[:, c] only.  Workgroup = (request, head, tile of 64 value columns), four
+// waves of 16 columns x 4 row groups.  A request's new tokens are walked in
+// order; operands are staged in LDS a chunk of tokens at a time, where all the
+// non-linearities are evaluated in parallel.
 #include "../ragged/ragged_common.h"
 
-constexpr int DR_COLS = 64;          // value columns per workgroup (one wave per row group)
+constexpr int DR_COLS = 64;          // value columns per workgroup
+constexpr int DR_RG = 4;             // row groups: a column's rows are dealt to 4 lanes of one wave
+constexpr int DR_NT = DR_COLS * DR_RG;
 constexpr int DR_MAX_RANK = 128;     // decay bottleneck
 
-template <typename T, int DMAX, int RG, int CH>
-__global__ __launch_bounds__(DR_COLS * RG) void delta_rule_kernel(
+// Thread mapping: wave w holds columns 16 w .. 16 w + 15 of the tile; inside a
+// wave lane = rg * 16 + c, so the four partial sums of a column sit in lanes
+// c, c + 16, c + 32, c + 48 and are reduced with two shuffles: the token loop
+// has no barrier.  Thread (column, rg) keeps rows rg * RPT .. rg * RPT + RPT - 1
+// of its column in registers.
+template <typename T, int DMAX, int CH>
+__global__ __launch_bounds__(DR_NT) void delta_rule_kernel(
     const T* __restrict__ proj, long stride, int r_off, int k_off, int v_off, int a_off, int w_off, int rank,
     const float* __restrict__ w2, const float* __restrict__ w0, const float* __restrict__ a_b,
     float* __restrict__ state, const int* __restrict__ cu, const int* __restrict__ slots, float* __restrict__ o,
-    int H, int D) {
-  constexpr int RPT = DMAX / RG;
-  constexpr int NT = DR_COLS * RG;
-  __shared__ float s_r[CH][DMAX], s_k[CH][DMAX], s_u[CH][DMAX], s_au[CH][DMAX], s_w[CH][DMAX];
+    int H, int D, int w2_in_lds) {
+  constexpr int RPT = DMAX / DR_RG;
+  __shared__ __align__(16) float s_r[CH][DMAX], s_k[CH][DMAX], s_u[CH][DMAX], s_au[CH][DMAX], s_w[CH][DMAX];
   __shared__ float s_v[CH][DR_COLS], s_b[CH][DR_MAX_RANK], s_inv[CH];
-  __shared__ float red1[2][RG][DR_COLS], red2[2][RG][DR_COLS];
+  extern __shared__ float s_w2[];                  // [rank][D] (transposed), when it fits
   const int r = blockIdx.x, hd = blockIdx.y, ct = blockIdx.z;
-  const int c = threadIdx.x % DR_COLS, rg = threadIdx.x / DR_COLS;     // a wave = one row group
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const int c = wave * 16 + (lane & 15), rg = lane >> 4;
   const int col = ct * DR_COLS + c;
   const bool colok = col < D;
   const long slot = slots[r];
@@ -36,74 +41,83 @@ __global__ __launch_bounds__(DR_COLS * RG) void delta_rule_kernel(
     const int row = rg * RPT + i;
     S[i] = (row < D && colok) ? sp[(long)row * D + col] : 0.f;
   }
+  // rows D .. DMAX-1 of the operand buffers are read by the token loop (against zero state): keep them zero
+  for (int i = threadIdx.x; i < CH * DMAX; i += DR_NT) {
+    (&s_r[0][0])[i] = 0.f; (&s_k[0][0])[i] = 0.f; (&s_u[0][0])[i] = 0.f; (&s_au[0][0])[i] = 0.f; (&s_w[0][0])[i] = 0.f;
+  }
+  if (w2_in_lds)
+    for (int i = threadIdx.x; i < D * rank; i += DR_NT) s_w2[(i % rank) * D + i / rank] = w2[(long)hd * D * rank + i];
+  __syncthreads();
   const int t0 = cu[r], t1 = cu[r + 1];
   const float decay_c = -0.60653065971263342f;     // -e^{-1/2}
-  int step = 0;
   for (int tc = t0; tc < t1; tc += CH) {
     const int nc = min(CH, t1 - tc);
-    for (int i = threadIdx.x; i < nc * rank; i += NT) {
+    for (int i = threadIdx.x; i < nc * rank; i += DR_NT) {
       const int tt = i / rank, j = i % rank;
       s_b[tt][j] = tanhf(ldf(proj + (long)(tc + tt) * stride + w_off + j));
     }
-    for (int i = threadIdx.x; i < nc * DR_COLS; i += NT) {
+    for (int i = threadIdx.x; i < nc * DR_COLS; i += DR_NT) {
       const int tt = i / DR_COLS, cc = ct * DR_COLS + i % DR_COLS;
       s_v[tt][i % DR_COLS] = (cc < D) ? ldf(proj + (long)(tc + tt) * stride + v_off + hd * D + cc) : 0.f;
     }
     __syncthreads();
-    for (int i = threadIdx.x; i < nc * D; i += NT) {
+    for (int i = threadIdx.x; i < nc * D; i += DR_NT) {
       const int tt = i / D, d = i % D, ch = hd * D + d;
       const T* row = proj + (long)(tc + tt) * stride;
       s_r[tt][d] = ldf(row + r_off + ch);
       s_k[tt][d] = ldf(row + k_off + ch);
       float z = w0[ch];
-      const float* w2r = w2 + (long)ch * rank;
-      for (int j = 0; j < rank; ++j) z += w2r[j] * s_b[tt][j];
+      if (w2_in_lds) {
+        for (int j = 0; j < rank; ++j) z += s_w2[j * D + d] * s_b[tt][j];
+      } else {
+        const float* w2r = w2 + (long)ch * rank;
+        for (int j = 0; j < rank; ++j) z += w2r[j] * s_b[tt][j];
+      }
       s_w[tt][d] = expf(decay_c * sigmoidf_(z));
       s_au[tt][d] = sigmoidf_(ldf(row + a_off + ch) + a_b[ch]);          // a for now, a * u below
     }
     __syncthreads();
-    for (int tt = rg; tt < nc; tt += RG) {          // one wave per token: squared norm of the key
+    for (int tt = wave; tt < nc; tt += DR_NT / WAVE) {   // one wave per token: squared norm of the key
       float ss = 0.f;
-      for (int d = c; d < D; d += DR_COLS) ss += s_k[tt][d] * s_k[tt][d];
+      for (int d = lane; d < D; d += WAVE) ss += s_k[tt][d] * s_k[tt][d];
       ss = wave_reduce_sum(ss);
-      if (c == 0) s_inv[tt] = 1.f / sqrtf(ss + 1e-6f);
+      if (lane == 0) s_inv[tt] = 1.f / sqrtf(ss + 1e-6f);
     }
     __syncthreads();
-    for (int i = threadIdx.x; i < nc * D; i += NT) {
+    for (int i = threadIdx.x; i < nc * D; i += DR_NT) {
       const int tt = i / D, d = i % D;
       const float u = s_k[tt][d] * s_inv[tt];
       s_u[tt][d] = u;
       s_au[tt][d] *= u;
     }
     __syncthreads();
-    for (int tt = 0; tt < nc; ++tt, ++step) {
+    for (int tt = 0; tt < nc; ++tt) {
       const float vv = s_v[tt][c];
-      float dot = 0.f;
+      const float* pu = &s_u[tt][rg * RPT];
+      const float* pw = &s_w[tt][rg * RPT];
+      const float* pa = &s_au[tt][rg * RPT];
+      const float* pk = &s_k[tt][rg * RPT];
+      const float* pr = &s_r[tt][rg * RPT];
+      float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
 #pragma unroll
-      for (int i = 0; i < RPT; ++i) dot += s_u[tt][rg * RPT + i] * S[i];     // rows >= D hold zeros in S
-      if constexpr (RG > 1) {
-        red1[step & 1][rg][c] = dot;
-        __syncthreads();
-        dot = 0.f;
-#pragma unroll
-        for (int g = 0; g < RG; ++g) dot += red1[step & 1][g][c];
+      for (int i = 0; i < RPT; i += 4) {
+        d0 += pu[i] * S[i]; d1 += pu[i + 1] * S[i + 1]; d2 += pu[i + 2] * S[i + 2]; d3 += pu[i + 3] * S[i + 3];
       }
-      float part = 0.f;
+      float dot = (d0 + d1) + (d2 + d3);
+      dot += __shfl_xor(dot, 16, 64);
+      dot += __shfl_xor(dot, 32, 64);
+      float p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;
 #pragma unroll
-      for (int i = 0; i < RPT; ++i) {
-        const int row = rg * RPT + i;
-        if (row < D) {
-          S[i] = s_w[tt][row] * S[i] - s_au[tt][row] * dot + s_k[tt][row] * vv;
-          part += s_r[tt][row] * S[i];
-        }
+      for (int i = 0; i < RPT; i += 4) {
+        S[i] = pw[i] * S[i] - pa[i] * dot + pk[i] * vv;
+        S[i + 1] = pw[i + 1] * S[i + 1] - pa[i + 1] * dot + pk[i + 1] * vv;
+        S[i + 2] = pw[i + 2] * S[i + 2] - pa[i + 2] * dot + pk[i + 2] * vv;
+        S[i + 3] = pw[i + 3] * S[i + 3] - pa[i + 3] * dot + pk[i + 3] * vv;
+        p0 += pr[i] * S[i]; p1 += pr[i + 1] * S[i + 1]; p2 += pr[i + 2] * S[i + 2]; p3 += pr[i + 3] * S[i + 3];
       }
-      if constexpr (RG > 1) {
-        red2[step & 1][rg][c] = part;
-        __syncthreads();
-        part = 0.f;
-#pragma unroll
-        for (int g = 0; g < RG; ++g) part += red2[step & 1][g][c];
-      }
+      float part = (p0 + p1) + (p2 + p3);
+      part += __shfl_xor(part, 16, 64);
+      part += __shfl_xor(part, 32, 64);
       if (rg == 0 && colok) o[((long)(tc + tt) * H + hd) * D + col] = part;
     }
     __syncthreads();                                // the chunk buffers are rewritten next
@@ -155,15 +169,20 @@ void delta_rule_scan(torch::Tensor proj, int64_t r_off, int64_t k_off, int64_t v
   auto o = torch::empty({T_, H, D}, proj.options().dtype(at::kFloat));
   auto stream = at::cuda::getCurrentHIPStream();
   const dim3 grid(R, (unsigned)H, (unsigned)((D + DR_COLS - 1) / DR_COLS));
-#define DR_LAUNCH(DMAX, RG, CH)                                                                                \
-  hipLaunchKernelGGL((delta_rule_kernel<T, DMAX, RG, CH>), grid, dim3(DR_COLS * RG), 0, stream,                \
+  // the head's second decay matrix is kept in LDS (transposed) when it fits beside the operand buffers
+  const size_t w2_bytes = (size_t)D * rank * sizeof(float);
+  const int w2_in_lds = w2_bytes <= 16 * 1024;
+  const size_t smem = w2_in_lds ? w2_bytes : 0;
+#define DR_LAUNCH(DMAX, CH)                                                                                    \
+  hipLaunchKernelGGL((delta_rule_kernel<T, DMAX, CH>), grid, dim3(DR_NT), smem, stream,                        \
       (const T*)proj.data_ptr(), (long)proj.stride(0), (int)r_off, (int)k_off, (int)v_off, (int)a_off,         \
       (int)w_off, (int)rank, w2.data_ptr<float>(), w0.data_ptr<float>(), a_b.data_ptr<float>(),                \
-      state.data_ptr<float>(), cu.data_ptr<int>(), slots.data_ptr<int>(), o.data_ptr<float>(), (int)H, (int)D)
+      state.data_ptr<float>(), cu.data_ptr<int>(), slots.data_ptr<int>(), o.data_ptr<float>(), (int)H, (int)D, \
+      w2_in_lds)
   RAGGED_DISPATCH(proj, {
-    if (D <= 64) DR_LAUNCH(64, 1, 16);
-    else if (D <= 128) DR_LAUNCH(128, 2, 16);
-    else DR_LAUNCH(256, 4, 8);
+    if (D <= 64) DR_LAUNCH(64, 16);
+    else if (D <= 128) DR_LAUNCH(128, 8);
+    else DR_LAUNCH(256, 8);
     const int TH = T_ * H;
     hipLaunchKernelGGL((delta_out_kernel<T>), dim3((TH + 3) / 4), dim3(256), 0, stream, o.data_ptr<float>(),
         (const T*)proj.data_ptr(), (long)proj.stride(0), (int)g_off, norm_w.data_ptr<float>(), (float)eps,

@@ -311,3 +311,19 @@ def moe_combine(down, inv, weights, shared, shared_gate, add):
                               shared_gate if shared is not None else _none(d),
                               add if add is not None else _none(d))
     return ref.moe_combine(down, inv, weights, shared, shared_gate, add)
+
+
+PAIR_PATH_MAX = 32      # (token, choice) pairs up to which every pair streams its expert's matrices itself
+
+
+def expert_pairs_ok(h, top, ff) -> bool:
+    """Steps with few pairs (decoding) skip the sort by expert: see csrc/hybrid/experts.hip."""
+    return (h.is_cuda and _H is not None and os.environ.get("MEGATRON_AMD_FORCE_REFERENCE", "0") != "1"
+            and h.shape[0] * top <= PAIR_PATH_MAX and h.shape[1] % 8 == 0 and ff % 8 == 0
+            and max(h.shape[1], ff) <= 16384)
+
+
+def expert_pairs(h, ids, w_gate_up, w_down, limit, alpha):
+    if _native_h(h):
+        return _H.expert_pairs(h, ids, w_gate_up, w_down, float(limit), float(alpha))
+    return ref.expert_pairs(h, ids, w_gate_up, w_down, limit, alpha)

@@ -401,3 +401,16 @@ def moe_combine(down, inv, weights, shared, shared_gate, add):
     if add is not None:
         y = y + add.float()
     return y
+
+
+def expert_pairs(h, ids, w_gate_up, w_down, limit, alpha):
+    """Every (token, choice) pair through its expert, rows in pair order
+    (token-major): clamped GLU of [gate; up] x, then the down product."""
+    T, K = ids.shape
+    out = torch.empty(T * K, h.shape[1], dtype=h.dtype, device=h.device)
+    for t in range(T):
+        for k in range(K):
+            e = int(ids[t, k])
+            y = clamped_glu(F.linear(h[t:t + 1], w_gate_up[e]), limit, alpha, h.dtype)
+            out[t * K + k] = F.linear(y, w_down[e])[0]
+    return out

@@ -43,6 +43,7 @@ RAGGED_SRC = [
 HYBRID_SRC = [
     "megatron_amd/ops/csrc/hybrid/bindings.cpp",
     "megatron_amd/ops/csrc/hybrid/rows.hip",
+    "megatron_amd/ops/csrc/hybrid/experts.hip",
     "megatron_amd/ops/csrc/hybrid/window_attention.hip",
     "megatron_amd/ops/csrc/hybrid/window_attention_mfma.hip",
     "megatron_amd/ops/csrc/hybrid/delta_rule.hip",

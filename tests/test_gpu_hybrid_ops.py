@@ -150,3 +150,18 @@ def test_glu_and_combine(dtype):
     _close(g[0], c[0], dtype, "glu")
     for a, b in zip(g[1:], c[1:]):
         _close(a, b, torch.float32, "combine")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_expert_pairs(dtype):
+    R = _need()
+
+    def run(dev, dt):
+        T, K, W, F_, E = 5, 3, 72, 40, 6
+        h = _rand((T, W), dt, dev)
+        ids = torch.stack([torch.randperm(E)[:K] for _ in range(T)]).to(torch.int32).to(dev)
+        wgu, wd = _rand((E, 2 * F_, W), dt, dev, 0.2), _rand((E, W, F_), dt, dev, 0.2)
+        return (R.expert_pairs(h, ids, wgu, wd, 1.2, 1.702),)
+
+    g, c = _both(run, dtype)
+    _close(g[0], c[0], dtype, "expert pairs")
