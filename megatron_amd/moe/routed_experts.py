@@ -11,7 +11,7 @@ y = g sigmoid(alpha g) (u + 1), output W_down y.
 Optional shared expert of the same form for every token, times
 sigmoid(w_sg . h); its gate row rides in the fp32 router GEMM.
 
-Step: one fp32 GEMM [router; shared gate], a routing kernel, then
+Step: one router kernel (fp32 logits of [router; shared gate], scores, selection), then
   * many pairs (prompt portions): the (token, choice) pairs are sorted by expert
     and each expert with work runs its gate/up and down products on its slice
     (vendor GEMMs; the pair counts are the step's one host read),
@@ -52,19 +52,18 @@ class RoutedExpertsMLP(nn.Module):
             self.ws_down = nn.Parameter(torch.zeros(hidden, shared_ff, dtype=dtype))
 
     def route(self, h: torch.Tensor):
-        logits = F.linear(h.float(), self.w_router)
-        ids, weights = R.moe_route(logits, self.experts, self.top, self.groups, self.keep, self.route_scale)
-        return logits, ids, weights
+        """-> (ids [T, top], weights [T, top], the shared expert's gate logit [T, 1] or [T, 0])"""
+        return R.moe_router(h, self.w_router, self.experts, self.top, self.groups, self.keep, self.route_scale)
 
     def forward(self, h: torch.Tensor, add: Optional[torch.Tensor] = None) -> torch.Tensor:
         """h [T, hidden] in the compute dtype -> fp32 [T, hidden] (+ add)."""
         T, K, E = h.shape[0], self.top, self.experts
-        logits, ids, weights = self.route(h)
+        ids, weights, extra = self.route(h)
         shared = gate = None
         if self.shared_ff:
             sy = R.clamped_glu(F.linear(h, self.ws_gate_up), self.shared_limit, self.alpha, h.dtype)
             shared = F.linear(sy, self.ws_down)
-            gate = logits[:, E].contiguous()
+            gate = extra.reshape(-1)
         if R.expert_pairs_ok(h, K, self.ff):
             # few pairs (decoding): each pair streams its expert's matrices, no sort, no host read
             down = R.expert_pairs(h, ids, self.w_gate_up, self.w_down, self.limit, self.alpha)

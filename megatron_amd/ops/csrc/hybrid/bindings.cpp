@@ -9,6 +9,8 @@ std::vector<torch::Tensor> residual_group_norm(torch::Tensor x, torch::Tensor y,
                                                int64_t groups, double eps, bool out_bf16);
 std::vector<torch::Tensor> moe_route(torch::Tensor logits, int64_t E, int64_t top, int64_t groups, int64_t keep,
                                      double scale);
+std::vector<torch::Tensor> moe_router(torch::Tensor h, torch::Tensor wr, int64_t E, int64_t top, int64_t groups,
+                                      int64_t keep, double scale);
 torch::Tensor clamped_glu(torch::Tensor gu, double limit, double alpha);
 torch::Tensor moe_combine(torch::Tensor down, torch::Tensor inv, torch::Tensor wts, torch::Tensor shared,
                           torch::Tensor gate, torch::Tensor add);
@@ -37,6 +39,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("embed_plain", &embed_plain);
   m.def("residual_group_norm", &residual_group_norm);
   m.def("moe_route", &moe_route);
+  m.def("moe_router", &moe_router);
   m.def("clamped_glu", &clamped_glu);
   m.def("moe_combine", &moe_combine);
   m.def("expert_pairs", &expert_pairs);

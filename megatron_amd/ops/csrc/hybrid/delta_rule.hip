@@ -13,9 +13,20 @@ constexpr int DR_RG = 4;             // row groups: a column's rows are dealt to
 constexpr int DR_NT = DR_COLS * DR_RG;
 constexpr int DR_MAX_RANK = 128;     // decay bottleneck
 
+// x summed over the four 16-lane rows of a wave, in every lane: two register
+// swaps between lane halves / neighbouring rows (VALU, no LDS round trip) and two adds
+__device__ __forceinline__ float sum_row_groups(float x) {
+  const int xi = __float_as_int(x);
+  auto a = __builtin_amdgcn_permlane32_swap(xi, xi, false, false);      // lanes l and l ^ 32 exchanged
+  const float y = __int_as_float(a[0]) + __int_as_float(a[1]);
+  const int yi = __float_as_int(y);
+  auto b = __builtin_amdgcn_permlane16_swap(yi, yi, false, false);      // rows r and r ^ 1 exchanged
+  return __int_as_float(b[0]) + __int_as_float(b[1]);
+}
+
 // Thread mapping: wave w holds columns 16 w .. 16 w + 15 of the tile; inside a
 // wave lane = rg * 16 + c, so the four partial sums of a column sit in lanes
-// c, c + 16, c + 32, c + 48 and are reduced with two shuffles: the token loop
+// c, c + 16, c + 32, c + 48 and are reduced with two register swaps: the token loop
 // has no barrier.  Thread (column, rg) keeps rows rg * RPT .. rg * RPT + RPT - 1
 // of its column in registers.
 template <typename T, int DMAX, int CH>
@@ -91,6 +102,7 @@ __global__ __launch_bounds__(DR_NT) void delta_rule_kernel(
       s_au[tt][d] *= u;
     }
     __syncthreads();
+#pragma unroll 2
     for (int tt = 0; tt < nc; ++tt) {
       const float vv = s_v[tt][c];
       const float* pu = &s_u[tt][rg * RPT];
@@ -103,9 +115,7 @@ __global__ __launch_bounds__(DR_NT) void delta_rule_kernel(
       for (int i = 0; i < RPT; i += 4) {
         d0 += pu[i] * S[i]; d1 += pu[i + 1] * S[i + 1]; d2 += pu[i + 2] * S[i + 2]; d3 += pu[i + 3] * S[i + 3];
       }
-      float dot = (d0 + d1) + (d2 + d3);
-      dot += __shfl_xor(dot, 16, 64);
-      dot += __shfl_xor(dot, 32, 64);
+      const float dot = sum_row_groups((d0 + d1) + (d2 + d3));
       float p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;
 #pragma unroll
       for (int i = 0; i < RPT; i += 4) {
@@ -115,9 +125,7 @@ __global__ __launch_bounds__(DR_NT) void delta_rule_kernel(
         S[i + 3] = pw[i + 3] * S[i + 3] - pa[i + 3] * dot + pk[i + 3] * vv;
         p0 += pr[i] * S[i]; p1 += pr[i + 1] * S[i + 1]; p2 += pr[i + 2] * S[i + 2]; p3 += pr[i + 3] * S[i + 3];
       }
-      float part = (p0 + p1) + (p2 + p3);
-      part += __shfl_xor(part, 16, 64);
-      part += __shfl_xor(part, 32, 64);
+      const float part = sum_row_groups((p0 + p1) + (p2 + p3));
       if (rg == 0 && colok) o[((long)(tc + tt) * H + hd) * D + col] = part;
     }
     __syncthreads();                                // the chunk buffers are rewritten next

@@ -177,6 +177,102 @@ std::vector<torch::Tensor> moe_route(torch::Tensor logits, int64_t E, int64_t to
 }
 
 // ---------------------------------------------------------------------------
+// router in one kernel: logits = W_r h in fp32 (W_r fp32, h from its storage
+// type), sigmoid scores, group-limited top-k, weights; rows beyond the experts
+// (a shared expert's gate vector) are returned as raw logits.
+// One workgroup per token: the waves take the rows of W_r in turn, one thread
+// selects from the scores in LDS.
+// ---------------------------------------------------------------------------
+constexpr int RF_MAX_ROWS = 512;
+
+template <typename T>
+__global__ __launch_bounds__(256) void moe_router_kernel(
+    const T* __restrict__ h, const float* __restrict__ wr, int W, int rows, int E, int top, int groups, int keep,
+    float scale, int* __restrict__ ids, float* __restrict__ wts, float* __restrict__ extra) {
+  extern __shared__ float xs[];                  // the token's input, fp32
+  __shared__ float sc[RF_MAX_ROWS];
+  const long t = blockIdx.x;
+  for (int i = threadIdx.x; i < W; i += 256) xs[i] = ldf(h + t * W + i);
+  __syncthreads();
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  for (int e = wave; e < rows; e += 4) {
+    const float* row = wr + (long)e * W;
+    float a = 0.f;
+    for (int d = lane; d < W; d += WAVE) a += row[d] * xs[d];
+    a = wave_reduce_sum(a);
+    if (lane == 0) {
+      if (e < E) sc[e] = sigmoidf_(a);
+      else extra[t * (rows - E) + (e - E)] = a;
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x != 0) return;
+  unsigned long long allowed = ~0ull;
+  const int per = E / groups;
+  if (groups > 1) {
+    float gsc[RT_MAX_GROUPS];
+    for (int g = 0; g < groups; ++g) {
+      float a = -1.f, b = -1.f;
+      for (int i = 0; i < per; ++i) {
+        const float s = sc[g * per + i];
+        if (s > a) { b = a; a = s; }
+        else if (s > b) b = s;
+      }
+      gsc[g] = a + (per > 1 ? b : 0.f);
+    }
+    allowed = 0ull;
+    for (int n = 0; n < keep; ++n) {
+      int best = -1;
+      float bv = -INFINITY;
+      for (int g = 0; g < groups; ++g)
+        if (!((allowed >> g) & 1ull) && gsc[g] > bv) { bv = gsc[g]; best = g; }
+      if (best >= 0) allowed |= 1ull << best;
+    }
+  }
+  float cs[RT_MAX_TOP];
+  int chosen[RT_MAX_TOP];
+  float sum = 0.f;
+  for (int n = 0; n < top; ++n) {
+    int best = -1;
+    float bv = -INFINITY;
+    for (int e = 0; e < E; ++e) {
+      if (groups > 1 && !((allowed >> (e / per)) & 1ull)) continue;
+      const float s = sc[e];
+      if (s > bv) { bv = s; best = e; }
+    }
+    chosen[n] = best < 0 ? 0 : best;
+    cs[n] = best < 0 ? 0.f : bv;
+    if (best >= 0) sc[best] = -2.f;               // taken
+    sum += cs[n];
+  }
+  for (int n = 0; n < top; ++n) {
+    ids[t * top + n] = chosen[n];
+    wts[t * top + n] = cs[n] / (sum + 1e-20f) * scale;
+  }
+}
+
+std::vector<torch::Tensor> moe_router(torch::Tensor h, torch::Tensor wr, int64_t E, int64_t top, int64_t groups,
+                                      int64_t keep, double scale) {
+  TORCH_CHECK(h.is_cuda() && h.dim() == 2 && h.is_contiguous());
+  check_f32(wr, "router weight");
+  const int T_ = h.size(0), W = h.size(1), rows = wr.size(0);
+  TORCH_CHECK(wr.dim() == 2 && wr.size(1) == W && E >= 1 && E <= rows && rows <= RF_MAX_ROWS);
+  TORCH_CHECK(top >= 1 && top <= RT_MAX_TOP && top <= E, "experts chosen per token");
+  TORCH_CHECK(groups >= 1 && groups <= RT_MAX_GROUPS && E % groups == 0 && keep >= 1 && keep <= groups);
+  TORCH_CHECK(groups == 1 || keep * (E / groups) >= top, "the kept groups hold fewer experts than are chosen");
+  TORCH_CHECK((size_t)W * sizeof(float) <= 64 * 1024, "row too wide for the router kernel");
+  auto ids = torch::empty({T_, top}, h.options().dtype(at::kInt));
+  auto wts = torch::empty({T_, top}, h.options().dtype(at::kFloat));
+  auto extra = torch::empty({T_, rows - E}, h.options().dtype(at::kFloat));
+  if (T_ == 0) return {ids, wts, extra};
+  auto stream = at::cuda::getCurrentHIPStream();
+  RAGGED_DISPATCH(h, hipLaunchKernelGGL((moe_router_kernel<T>), dim3(T_), dim3(256), (size_t)W * sizeof(float), stream,
+      (const T*)h.data_ptr(), wr.data_ptr<float>(), W, rows, (int)E, (int)top, (int)groups, (int)keep, (float)scale,
+      ids.data_ptr<int>(), wts.data_ptr<float>(), extra.data_ptr<float>()));
+  return {ids, wts, extra};
+}
+
+// ---------------------------------------------------------------------------
 // y = g sigmoid(alpha g) (u + 1),  g = min(gate, limit), u = clamp(up, -limit, limit)
 // ---------------------------------------------------------------------------
 template <typename T>

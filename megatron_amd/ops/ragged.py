@@ -327,3 +327,10 @@ def expert_pairs(h, ids, w_gate_up, w_down, limit, alpha):
     if _native_h(h):
         return _H.expert_pairs(h, ids, w_gate_up, w_down, float(limit), float(alpha))
     return ref.expert_pairs(h, ids, w_gate_up, w_down, limit, alpha)
+
+
+def moe_router(h, w_router, experts, top, groups, keep, scale):
+    """-> (ids [T, top] int32, weights [T, top] fp32, raw logits of the rows beyond the experts)"""
+    if _native_h(h) and h.shape[1] <= 16384 and w_router.shape[0] <= 512:
+        return _H.moe_router(h, w_router, int(experts), int(top), int(groups), int(keep), float(scale))
+    return ref.moe_router(h, w_router, experts, top, groups, keep, scale)

@@ -414,3 +414,11 @@ def expert_pairs(h, ids, w_gate_up, w_down, limit, alpha):
             y = clamped_glu(F.linear(h[t:t + 1], w_gate_up[e]), limit, alpha, h.dtype)
             out[t * K + k] = F.linear(y, w_down[e])[0]
     return out
+
+
+def moe_router(h, w_router, experts, top, groups, keep, scale):
+    """Router in one call: fp32 logits of all rows of w_router (the rows beyond
+    ``experts`` are returned raw), then moe_route.  -> (ids, weights, extra [T, rows - experts])"""
+    logits = F.linear(h.float(), w_router.float())
+    ids, weights = moe_route(logits, experts, top, groups, keep, scale)
+    return ids, weights, logits[:, experts:].contiguous()

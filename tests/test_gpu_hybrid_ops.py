@@ -165,3 +165,23 @@ def test_expert_pairs(dtype):
 
     g, c = _both(run, dtype)
     _close(g[0], c[0], dtype, "expert pairs")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("cfg", [(12, 4, 4, 3, 1), (8, 2, 1, 1, 0), (64, 8, 8, 4, 1), (5, 5, 1, 1, 2)])
+def test_moe_router_fused(dtype, cfg):
+    R = _need()
+    E, top, groups, keep, extra = cfg
+
+    def run(dev, dt):
+        h = _rand((23, 88), dt, dev)
+        wr = _rand((E + extra, 88), torch.float32, dev, 0.4)
+        ids, w, ex = R.moe_router(h, wr, E, top, groups, keep, 1.5)
+        order = ids.long().argsort(dim=1)
+        return ids.long().gather(1, order).float(), w.gather(1, order), ex
+
+    g, c = _both(run, dtype)
+    assert torch.equal(g[0].cpu(), c[0]), "chosen experts"
+    _close(g[1], c[1], torch.float32, "weights")
+    if extra:
+        _close(g[2], c[2], torch.float32, "extra logits")
