@@ -2,15 +2,17 @@
 //   S <- diag(w) S - (a u)(u^T S) + k v^T ,  o = S^T r      (per head; both terms read the old S)
 //   w = exp(-e^{-1/2} sigmoid(W2 tanh(b) + w0)),  a = sigmoid(a_pre + a_b),  u = k / sqrt(sum k^2 + 1e-6)
 // The update is independent per value column: S[:, c] needs u . S[:, c] and
-// r . S[:, c] only.  Workgroup = (request, head, tile of 64 value columns), four
-// waves of 16 columns x 4 row groups.  A request's new tokens are walked in
-// order; operands are staged in LDS a chunk of tokens at a time, where all the
-// non-linearities are evaluated in parallel.
+// r . S[:, c] only.  Workgroup = (request, head, tile of 64 value columns).  A
+// request's new tokens are walked in order by four consumer waves while four
+// producer waves prepare the next chunk's operands (all the non-linearities)
+// in LDS.
 #include "../ragged/ragged_common.h"
 
 constexpr int DR_COLS = 64;          // value columns per workgroup
 constexpr int DR_RG = 4;             // row groups: a column's rows are dealt to 4 lanes of one wave
-constexpr int DR_NT = DR_COLS * DR_RG;
+constexpr int DR_CONS = DR_COLS * DR_RG;        // consumer threads (4 waves): the token loop
+constexpr int DR_PROD_WAVES = 4;                // producer waves: operand staging for the next chunk
+constexpr int DR_NT = DR_CONS + DR_PROD_WAVES * WAVE;
 constexpr int DR_MAX_RANK = 128;     // decay bottleneck
 
 // x summed over the four 16-lane rows of a wave, in every lane: two register
@@ -24,11 +26,20 @@ __device__ __forceinline__ float sum_row_groups(float x) {
   return __int_as_float(b[0]) + __int_as_float(b[1]);
 }
 
-// Thread mapping: wave w holds columns 16 w .. 16 w + 15 of the tile; inside a
-// wave lane = rg * 16 + c, so the four partial sums of a column sit in lanes
-// c, c + 16, c + 32, c + 48 and are reduced with two register swaps: the token loop
-// has no barrier.  Thread (column, rg) keeps rows rg * RPT .. rg * RPT + RPT - 1
-// of its column in registers.
+__device__ __forceinline__ float lane_value(float x, int src_lane) {     // src_lane is wave-uniform
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), src_lane));
+}
+
+// Eight waves with two roles.  Consumer waves 0-3 run the token loop: wave w
+// holds columns 16 w .. 16 w + 15 of the tile; inside a wave lane = rg * 16 + c,
+// so the four partial sums of a column sit in lanes c, c + 16, c + 32, c + 48 and
+// are reduced with two register swaps: the token loop has no barrier.  Thread
+// (column, rg) keeps rows rg * RPT .. rg * RPT + RPT - 1 of its column in registers.
+// Producer waves 4-7 stage the operands of the NEXT chunk of tokens into the
+// other half of a double buffer meanwhile, one wave per token, lanes over the
+// channels: projections read, bottleneck tanh and second decay matrix, decay,
+// removal rate, unit key; values pass between lanes in registers, so a
+// producer needs no barrier either.  One workgroup barrier per chunk.
 template <typename T, int DMAX, int CH>
 __global__ __launch_bounds__(DR_NT) void delta_rule_kernel(
     const T* __restrict__ proj, long stride, int r_off, int k_off, int v_off, int a_off, int w_off, int rank,
@@ -36,104 +47,136 @@ __global__ __launch_bounds__(DR_NT) void delta_rule_kernel(
     float* __restrict__ state, const int* __restrict__ cu, const int* __restrict__ slots, float* __restrict__ o,
     int H, int D, int w2_in_lds) {
   constexpr int RPT = DMAX / DR_RG;
-  __shared__ __align__(16) float s_r[CH][DMAX], s_k[CH][DMAX], s_u[CH][DMAX], s_au[CH][DMAX], s_w[CH][DMAX];
-  __shared__ float s_v[CH][DR_COLS], s_b[CH][DR_MAX_RANK], s_inv[CH];
+  constexpr int EPL = DMAX / WAVE;                 // channels per producer lane
+  __shared__ __align__(16) float s_r[2][CH][DMAX], s_k[2][CH][DMAX], s_u[2][CH][DMAX], s_au[2][CH][DMAX],
+      s_w[2][CH][DMAX];
+  __shared__ float s_v[2][CH][DR_COLS];
   extern __shared__ float s_w2[];                  // [rank][D] (transposed), when it fits
   const int r = blockIdx.x, hd = blockIdx.y, ct = blockIdx.z;
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-  const int c = wave * 16 + (lane & 15), rg = lane >> 4;
+  const bool producer = wave >= DR_CONS / WAVE;
+  const int t0 = cu[r], t1 = cu[r + 1];
+  const int nchunks = (t1 - t0 + CH - 1) / CH;
+  if (w2_in_lds)
+    for (int i = threadIdx.x; i < D * rank; i += DR_NT) s_w2[(i % rank) * D + i / rank] = w2[(long)hd * D * rank + i];
+  __syncthreads();
+
+  // ---- producer: operands of chunk ci into buffer b (rows D .. DMAX-1 are written as zeros) ----
+  auto stage = [&](int ci, int b) {
+    const int tc = t0 + ci * CH;
+    const int nc = min(CH, t1 - tc);
+    const float decay_c = -0.60653065971263342f;   // -e^{-1/2}
+    for (int tt = wave - DR_CONS / WAVE; tt < nc; tt += DR_PROD_WAVES) {
+      const T* row = proj + (long)(tc + tt) * stride;
+      float tb0 = 0.f, tb1 = 0.f;                  // tanh of the bottleneck, entry j in lane j % 64
+      if (lane < rank) tb0 = tanhf(ldf(row + w_off + lane));
+      if (lane + WAVE < rank) tb1 = tanhf(ldf(row + w_off + lane + WAVE));
+      float kk[EPL], rr[EPL], aa[EPL], zz[EPL];
+      float ss = 0.f;
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) {
+        const int d = lane + WAVE * e;
+        const bool ok = d < D;
+        const int ch = hd * D + (ok ? d : 0);
+        kk[e] = ok ? ldf(row + k_off + ch) : 0.f;
+        rr[e] = ok ? ldf(row + r_off + ch) : 0.f;
+        aa[e] = ok ? sigmoidf_(ldf(row + a_off + ch) + a_b[ch]) : 0.f;
+        zz[e] = ok ? w0[ch] : 0.f;
+        ss += kk[e] * kk[e];
+      }
+      const int r0 = min(rank, WAVE);
+      for (int j = 0; j < r0; ++j) {
+        const float tj = lane_value(tb0, j);
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+          const int d = lane + WAVE * e;
+          if (d < D) zz[e] += (w2_in_lds ? s_w2[j * D + d] : w2[(long)(hd * D + d) * rank + j]) * tj;
+        }
+      }
+      for (int j = WAVE; j < rank; ++j) {
+        const float tj = lane_value(tb1, j - WAVE);
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+          const int d = lane + WAVE * e;
+          if (d < D) zz[e] += (w2_in_lds ? s_w2[j * D + d] : w2[(long)(hd * D + d) * rank + j]) * tj;
+        }
+      }
+      const float inv = 1.f / sqrtf(wave_reduce_sum(ss) + 1e-6f);
+#pragma unroll
+      for (int e = 0; e < EPL; ++e) {
+        const int d = lane + WAVE * e;
+        const bool ok = d < D;
+        const float u = kk[e] * inv;
+        s_r[b][tt][d] = rr[e];
+        s_k[b][tt][d] = kk[e];
+        s_u[b][tt][d] = u;
+        s_au[b][tt][d] = aa[e] * u;
+        s_w[b][tt][d] = ok ? expf(decay_c * sigmoidf_(zz[e])) : 0.f;
+      }
+      const int cc = ct * DR_COLS + lane;
+      s_v[b][tt][lane] = (cc < D) ? ldf(row + v_off + hd * D + cc) : 0.f;
+    }
+  };
+
+  // ---- consumer state ----
+  const int c = (wave & 3) * 16 + (lane & 15), rg = lane >> 4;
   const int col = ct * DR_COLS + c;
   const bool colok = col < D;
   const long slot = slots[r];
   float* sp = state + ((slot * H + hd) * D) * (long)D;
   float S[RPT];
+  if (!producer) {
 #pragma unroll
-  for (int i = 0; i < RPT; ++i) {
-    const int row = rg * RPT + i;
-    S[i] = (row < D && colok) ? sp[(long)row * D + col] : 0.f;
+    for (int i = 0; i < RPT; ++i) {
+      const int row = rg * RPT + i;
+      S[i] = (row < D && colok) ? sp[(long)row * D + col] : 0.f;
+    }
+  } else if (nchunks > 0) {
+    stage(0, 0);
   }
-  // rows D .. DMAX-1 of the operand buffers are read by the token loop (against zero state): keep them zero
-  for (int i = threadIdx.x; i < CH * DMAX; i += DR_NT) {
-    (&s_r[0][0])[i] = 0.f; (&s_k[0][0])[i] = 0.f; (&s_u[0][0])[i] = 0.f; (&s_au[0][0])[i] = 0.f; (&s_w[0][0])[i] = 0.f;
-  }
-  if (w2_in_lds)
-    for (int i = threadIdx.x; i < D * rank; i += DR_NT) s_w2[(i % rank) * D + i / rank] = w2[(long)hd * D * rank + i];
   __syncthreads();
-  const int t0 = cu[r], t1 = cu[r + 1];
-  const float decay_c = -0.60653065971263342f;     // -e^{-1/2}
-  for (int tc = t0; tc < t1; tc += CH) {
-    const int nc = min(CH, t1 - tc);
-    for (int i = threadIdx.x; i < nc * rank; i += DR_NT) {
-      const int tt = i / rank, j = i % rank;
-      s_b[tt][j] = tanhf(ldf(proj + (long)(tc + tt) * stride + w_off + j));
-    }
-    for (int i = threadIdx.x; i < nc * DR_COLS; i += DR_NT) {
-      const int tt = i / DR_COLS, cc = ct * DR_COLS + i % DR_COLS;
-      s_v[tt][i % DR_COLS] = (cc < D) ? ldf(proj + (long)(tc + tt) * stride + v_off + hd * D + cc) : 0.f;
-    }
-    __syncthreads();
-    for (int i = threadIdx.x; i < nc * D; i += DR_NT) {
-      const int tt = i / D, d = i % D, ch = hd * D + d;
-      const T* row = proj + (long)(tc + tt) * stride;
-      s_r[tt][d] = ldf(row + r_off + ch);
-      s_k[tt][d] = ldf(row + k_off + ch);
-      float z = w0[ch];
-      if (w2_in_lds) {
-        for (int j = 0; j < rank; ++j) z += s_w2[j * D + d] * s_b[tt][j];
-      } else {
-        const float* w2r = w2 + (long)ch * rank;
-        for (int j = 0; j < rank; ++j) z += w2r[j] * s_b[tt][j];
-      }
-      s_w[tt][d] = expf(decay_c * sigmoidf_(z));
-      s_au[tt][d] = sigmoidf_(ldf(row + a_off + ch) + a_b[ch]);          // a for now, a * u below
-    }
-    __syncthreads();
-    for (int tt = wave; tt < nc; tt += DR_NT / WAVE) {   // one wave per token: squared norm of the key
-      float ss = 0.f;
-      for (int d = lane; d < D; d += WAVE) ss += s_k[tt][d] * s_k[tt][d];
-      ss = wave_reduce_sum(ss);
-      if (lane == 0) s_inv[tt] = 1.f / sqrtf(ss + 1e-6f);
-    }
-    __syncthreads();
-    for (int i = threadIdx.x; i < nc * D; i += DR_NT) {
-      const int tt = i / D, d = i % D;
-      const float u = s_k[tt][d] * s_inv[tt];
-      s_u[tt][d] = u;
-      s_au[tt][d] *= u;
-    }
-    __syncthreads();
+  for (int ci = 0; ci < nchunks; ++ci) {
+    const int b = ci & 1;
+    if (producer) {
+      if (ci + 1 < nchunks) stage(ci + 1, b ^ 1);
+    } else {
+      const int tc = t0 + ci * CH;
+      const int nc = min(CH, t1 - tc);
 #pragma unroll 2
-    for (int tt = 0; tt < nc; ++tt) {
-      const float vv = s_v[tt][c];
-      const float* pu = &s_u[tt][rg * RPT];
-      const float* pw = &s_w[tt][rg * RPT];
-      const float* pa = &s_au[tt][rg * RPT];
-      const float* pk = &s_k[tt][rg * RPT];
-      const float* pr = &s_r[tt][rg * RPT];
-      float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
+      for (int tt = 0; tt < nc; ++tt) {
+        const float vv = s_v[b][tt][c];
+        const float* pu = &s_u[b][tt][rg * RPT];
+        const float* pw = &s_w[b][tt][rg * RPT];
+        const float* pa = &s_au[b][tt][rg * RPT];
+        const float* pk = &s_k[b][tt][rg * RPT];
+        const float* pr = &s_r[b][tt][rg * RPT];
+        float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
 #pragma unroll
-      for (int i = 0; i < RPT; i += 4) {
-        d0 += pu[i] * S[i]; d1 += pu[i + 1] * S[i + 1]; d2 += pu[i + 2] * S[i + 2]; d3 += pu[i + 3] * S[i + 3];
-      }
-      const float dot = sum_row_groups((d0 + d1) + (d2 + d3));
-      float p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;
+        for (int i = 0; i < RPT; i += 4) {
+          d0 += pu[i] * S[i]; d1 += pu[i + 1] * S[i + 1]; d2 += pu[i + 2] * S[i + 2]; d3 += pu[i + 3] * S[i + 3];
+        }
+        const float dot = sum_row_groups((d0 + d1) + (d2 + d3));
+        float p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;
 #pragma unroll
-      for (int i = 0; i < RPT; i += 4) {
-        S[i] = pw[i] * S[i] - pa[i] * dot + pk[i] * vv;
-        S[i + 1] = pw[i + 1] * S[i + 1] - pa[i + 1] * dot + pk[i + 1] * vv;
-        S[i + 2] = pw[i + 2] * S[i + 2] - pa[i + 2] * dot + pk[i + 2] * vv;
-        S[i + 3] = pw[i + 3] * S[i + 3] - pa[i + 3] * dot + pk[i + 3] * vv;
-        p0 += pr[i] * S[i]; p1 += pr[i + 1] * S[i + 1]; p2 += pr[i + 2] * S[i + 2]; p3 += pr[i + 3] * S[i + 3];
+        for (int i = 0; i < RPT; i += 4) {
+          S[i] = pw[i] * S[i] - pa[i] * dot + pk[i] * vv;
+          S[i + 1] = pw[i + 1] * S[i + 1] - pa[i + 1] * dot + pk[i + 1] * vv;
+          S[i + 2] = pw[i + 2] * S[i + 2] - pa[i + 2] * dot + pk[i + 2] * vv;
+          S[i + 3] = pw[i + 3] * S[i + 3] - pa[i + 3] * dot + pk[i + 3] * vv;
+          p0 += pr[i] * S[i]; p1 += pr[i + 1] * S[i + 1]; p2 += pr[i + 2] * S[i + 2]; p3 += pr[i + 3] * S[i + 3];
+        }
+        const float part = sum_row_groups((p0 + p1) + (p2 + p3));
+        if (rg == 0 && colok) o[((long)(tc + tt) * H + hd) * D + col] = part;
       }
-      const float part = sum_row_groups((p0 + p1) + (p2 + p3));
-      if (rg == 0 && colok) o[((long)(tc + tt) * H + hd) * D + col] = part;
     }
-    __syncthreads();                                // the chunk buffers are rewritten next
+    __syncthreads();
   }
+  if (!producer) {
 #pragma unroll
-  for (int i = 0; i < RPT; ++i) {
-    const int row = rg * RPT + i;
-    if (row < D && colok) sp[(long)row * D + col] = S[i];
+    for (int i = 0; i < RPT; ++i) {
+      const int row = rg * RPT + i;
+      if (row < D && colok) sp[(long)row * D + col] = S[i];
+    }
   }
 }
 
@@ -188,9 +231,9 @@ void delta_rule_scan(torch::Tensor proj, int64_t r_off, int64_t k_off, int64_t v
       state.data_ptr<float>(), cu.data_ptr<int>(), slots.data_ptr<int>(), o.data_ptr<float>(), (int)H, (int)D, \
       w2_in_lds)
   RAGGED_DISPATCH(proj, {
-    if (D <= 64) DR_LAUNCH(64, 16);
+    if (D <= 64) DR_LAUNCH(64, 8);
     else if (D <= 128) DR_LAUNCH(128, 8);
-    else DR_LAUNCH(256, 8);
+    else DR_LAUNCH(256, 4);
     const int TH = T_ * H;
     hipLaunchKernelGGL((delta_out_kernel<T>), dim3((TH + 3) / 4), dim3(256), 0, stream, o.data_ptr<float>(),
         (const T*)proj.data_ptr(), (long)proj.stride(0), (int)g_off, norm_w.data_ptr<float>(), (float)eps,

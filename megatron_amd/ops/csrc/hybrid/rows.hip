@@ -180,26 +180,35 @@ std::vector<torch::Tensor> moe_route(torch::Tensor logits, int64_t E, int64_t to
 // router in one kernel: logits = W_r h in fp32 (W_r fp32, h from its storage
 // type), sigmoid scores, group-limited top-k, weights; rows beyond the experts
 // (a shared expert's gate vector) are returned as raw logits.
-// One workgroup per token: the waves take the rows of W_r in turn, one thread
-// selects from the scores in LDS.
+// One workgroup per token: its eight waves take the rows of W_r in turn (16 B
+// loads, four partial sums), one thread selects from the scores in LDS.
 // ---------------------------------------------------------------------------
 constexpr int RF_MAX_ROWS = 512;
 
+constexpr int RF_THREADS = 512;
+
 template <typename T>
-__global__ __launch_bounds__(256) void moe_router_kernel(
+__global__ __launch_bounds__(RF_THREADS) void moe_router_kernel(
     const T* __restrict__ h, const float* __restrict__ wr, int W, int rows, int E, int top, int groups, int keep,
     float scale, int* __restrict__ ids, float* __restrict__ wts, float* __restrict__ extra) {
-  extern __shared__ float xs[];                  // the token's input, fp32
+  extern __shared__ __align__(16) float xs[];    // the token's input, fp32
   __shared__ float sc[RF_MAX_ROWS];
   const long t = blockIdx.x;
-  for (int i = threadIdx.x; i < W; i += 256) xs[i] = ldf(h + t * W + i);
+  for (int i = threadIdx.x; i < W; i += RF_THREADS) xs[i] = ldf(h + t * W + i);
   __syncthreads();
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-  for (int e = wave; e < rows; e += 4) {
+  const int W4 = (W % 4 == 0) ? W : 0;           // 16 B pieces when rows stay aligned
+  for (int e = wave; e < rows; e += RF_THREADS / WAVE) {
     const float* row = wr + (long)e * W;
-    float a = 0.f;
-    for (int d = lane; d < W; d += WAVE) a += row[d] * xs[d];
-    a = wave_reduce_sum(a);
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+#pragma unroll 4
+    for (int d = lane * 4; d < W4; d += WAVE * 4) {
+      const float4v w = *reinterpret_cast<const float4v*>(row + d);
+      const float4v x = *reinterpret_cast<const float4v*>(xs + d);
+      a0 += w[0] * x[0]; a1 += w[1] * x[1]; a2 += w[2] * x[2]; a3 += w[3] * x[3];
+    }
+    for (int d = W4 + lane; d < W; d += WAVE) a0 += row[d] * xs[d];
+    const float a = wave_reduce_sum((a0 + a1) + (a2 + a3));
     if (lane == 0) {
       if (e < E) sc[e] = sigmoidf_(a);
       else extra[t * (rows - E) + (e - E)] = a;
@@ -266,7 +275,7 @@ std::vector<torch::Tensor> moe_router(torch::Tensor h, torch::Tensor wr, int64_t
   auto extra = torch::empty({T_, rows - E}, h.options().dtype(at::kFloat));
   if (T_ == 0) return {ids, wts, extra};
   auto stream = at::cuda::getCurrentHIPStream();
-  RAGGED_DISPATCH(h, hipLaunchKernelGGL((moe_router_kernel<T>), dim3(T_), dim3(256), (size_t)W * sizeof(float), stream,
+  RAGGED_DISPATCH(h, hipLaunchKernelGGL((moe_router_kernel<T>), dim3(T_), dim3(RF_THREADS), (size_t)W * sizeof(float), stream,
       (const T*)h.data_ptr(), wr.data_ptr<float>(), W, rows, (int)E, (int)top, (int)groups, (int)keep, (float)scale,
       ids.data_ptr<int>(), wts.data_ptr<float>(), extra.data_ptr<float>()));
   return {ids, wts, extra};
