@@ -2,46 +2,44 @@
 //   S <- diag(w) S - (a u)(u^T S) + k v^T ,  o = S^T r      (per head; both terms read the old S)
 //   w = exp(-e^{-1/2} sigmoid(W2 tanh(b) + w0)),  a = sigmoid(a_pre + a_b),  u = k / sqrt(sum k^2 + 1e-6)
 // The update is independent per value column: S[:, c] needs u . S[:, c] and
-// r . S[:, c] only.  Workgroup = (request, head, tile of 64 value columns).  A
-// request's new tokens are walked in order by four consumer waves while four
+// r . S[:, c] only.  Workgroup = (request, head, tile of 16 value columns).  A
+// request's new tokens are walked in order by four consumer waves while the
 // producer waves prepare the next chunk's operands (all the non-linearities)
 // in LDS.
 #include "../ragged/ragged_common.h"
 
-constexpr int DR_COLS = 64;          // value columns per workgroup
-constexpr int DR_RG = 4;             // row groups: a column's rows are dealt to 4 lanes of one wave
+constexpr int DR_COLS = 16;          // value columns per workgroup
+constexpr int DR_RG = 16;            // row groups: a column's rows are dealt to the 16 lanes of one wave row
 constexpr int DR_CONS = DR_COLS * DR_RG;        // consumer threads (4 waves): the token loop
-constexpr int DR_PROD_WAVES = 4;                // producer waves: operand staging for the next chunk
-constexpr int DR_NT = DR_CONS + DR_PROD_WAVES * WAVE;
 constexpr int DR_MAX_RANK = 128;     // decay bottleneck
 
-// x summed over the four 16-lane rows of a wave, in every lane: two register
-// swaps between lane halves / neighbouring rows (VALU, no LDS round trip) and two adds
-__device__ __forceinline__ float sum_row_groups(float x) {
-  const int xi = __float_as_int(x);
-  auto a = __builtin_amdgcn_permlane32_swap(xi, xi, false, false);      // lanes l and l ^ 32 exchanged
-  const float y = __int_as_float(a[0]) + __int_as_float(a[1]);
-  const int yi = __float_as_int(y);
-  auto b = __builtin_amdgcn_permlane16_swap(yi, yi, false, false);      // rows r and r ^ 1 exchanged
-  return __int_as_float(b[0]) + __int_as_float(b[1]);
+// x summed over the 16 lanes of its wave row, in every lane: four rotations inside
+// the row (DPP modifiers of the adds: VALU only, no LDS round trip)
+__device__ __forceinline__ float sum_row(float x) {
+  x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x128, 0xf, 0xf, false));   // row_ror:8
+  x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x124, 0xf, 0xf, false));   // row_ror:4
+  x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x122, 0xf, 0xf, false));   // row_ror:2
+  x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x121, 0xf, 0xf, false));   // row_ror:1
+  return x;
 }
 
 __device__ __forceinline__ float lane_value(float x, int src_lane) {     // src_lane is wave-uniform
   return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), src_lane));
 }
 
-// Eight waves with two roles.  Consumer waves 0-3 run the token loop: wave w
-// holds columns 16 w .. 16 w + 15 of the tile; inside a wave lane = rg * 16 + c,
-// so the four partial sums of a column sit in lanes c, c + 16, c + 32, c + 48 and
-// are reduced with two register swaps: the token loop has no barrier.  Thread
-// (column, rg) keeps rows rg * RPT .. rg * RPT + RPT - 1 of its column in registers.
-// Producer waves 4-7 stage the operands of the NEXT chunk of tokens into the
-// other half of a double buffer meanwhile, one wave per token, lanes over the
+// Waves with two roles.  Consumer waves 0-3 run the token loop: wave w holds
+// columns 4 w .. 4 w + 3 of the tile; inside a wave lane = 16 cw + rg owns rows
+// rg * RPT .. rg * RPT + RPT - 1 of column 4 w + cw in registers; the sixteen partial
+// sums of a column sit in one wave row and are reduced in registers: the token
+// loop has no barrier and a few dozen instructions per token.
+// Producer waves stage the operands of the NEXT chunk of tokens into the other
+// half of a double buffer meanwhile, one wave per token, lanes over the
 // channels: projections read, bottleneck tanh and second decay matrix, decay,
 // removal rate, unit key; values pass between lanes in registers, so a
-// producer needs no barrier either.  One workgroup barrier per chunk.
-template <typename T, int DMAX, int CH>
-__global__ __launch_bounds__(DR_NT) void delta_rule_kernel(
+// producer needs no barrier either.  One workgroup barrier per chunk.  (The
+// column tiles of a head repeat the staging; they run on different CUs.)
+template <typename T, int DMAX, int CH, int PW>
+__global__ __launch_bounds__(DR_CONS + PW * WAVE) void delta_rule_kernel(
     const T* __restrict__ proj, long stride, int r_off, int k_off, int v_off, int a_off, int w_off, int rank,
     const float* __restrict__ w2, const float* __restrict__ w0, const float* __restrict__ a_b,
     float* __restrict__ state, const int* __restrict__ cu, const int* __restrict__ slots, float* __restrict__ o,
@@ -54,72 +52,99 @@ __global__ __launch_bounds__(DR_NT) void delta_rule_kernel(
   extern __shared__ float s_w2[];                  // [rank][D] (transposed), when it fits
   const int r = blockIdx.x, hd = blockIdx.y, ct = blockIdx.z;
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-  const bool producer = wave >= DR_CONS / WAVE;
+  const bool producer = wave >= DR_CONS / WAVE;   // wave-uniform
   const int t0 = cu[r], t1 = cu[r + 1];
   const int nchunks = (t1 - t0 + CH - 1) / CH;
   if (w2_in_lds)
-    for (int i = threadIdx.x; i < D * rank; i += DR_NT) s_w2[(i % rank) * D + i / rank] = w2[(long)hd * D * rank + i];
+    for (int i = threadIdx.x; i < D * rank; i += DR_CONS + PW * WAVE) s_w2[(i % rank) * D + i / rank] = w2[(long)hd * D * rank + i];
   __syncthreads();
 
-  // ---- producer: operands of chunk ci into buffer b (rows D .. DMAX-1 are written as zeros) ----
-  auto stage = [&](int ci, int b) {
+  // ---- producer: a wave owns tokens pw, pw + PW, ... of a chunk.  load() only issues the
+  // global reads of a chunk into registers; finish() does the arithmetic and writes buffer b
+  // (rows D .. DMAX-1 as zeros).  The reads of chunk ci + 2 are issued right after chunk ci + 1
+  // was finished, so their latency passes while the consumers walk chunk ci.
+  constexpr int TPW = CH / PW;
+  static_assert(CH % PW == 0, "a chunk is dealt evenly to the producer waves");
+  const int pw = wave - DR_CONS / WAVE;
+  float kk[TPW][EPL], rr[TPW][EPL], ar[TPW][EPL], b0[TPW], b1[TPW], vr[TPW];
+  auto load = [&](int ci) {
+    const int tc = t0 + ci * CH;
+    const int nc = min(CH, t1 - tc);
+#pragma unroll
+    for (int s = 0; s < TPW; ++s) {
+      const int tt = pw + PW * s;
+      if (tt < nc) {
+        const T* row = proj + (long)(tc + tt) * stride;
+        b0[s] = (lane < rank) ? ldf(row + w_off + lane) : 0.f;
+        b1[s] = (lane + WAVE < rank) ? ldf(row + w_off + lane + WAVE) : 0.f;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+          const int d = lane + WAVE * e;
+          const bool ok = d < D;
+          const int ch = hd * D + (ok ? d : 0);
+          kk[s][e] = ok ? ldf(row + k_off + ch) : 0.f;
+          rr[s][e] = ok ? ldf(row + r_off + ch) : 0.f;
+          ar[s][e] = ok ? ldf(row + a_off + ch) : 0.f;
+        }
+        const int cc = ct * DR_COLS + lane;
+        vr[s] = (lane < DR_COLS && cc < D) ? ldf(row + v_off + hd * D + cc) : 0.f;
+      }
+    }
+  };
+  auto finish = [&](int ci, int b) {
     const int tc = t0 + ci * CH;
     const int nc = min(CH, t1 - tc);
     const float decay_c = -0.60653065971263342f;   // -e^{-1/2}
-    for (int tt = wave - DR_CONS / WAVE; tt < nc; tt += DR_PROD_WAVES) {
-      const T* row = proj + (long)(tc + tt) * stride;
-      float tb0 = 0.f, tb1 = 0.f;                  // tanh of the bottleneck, entry j in lane j % 64
-      if (lane < rank) tb0 = tanhf(ldf(row + w_off + lane));
-      if (lane + WAVE < rank) tb1 = tanhf(ldf(row + w_off + lane + WAVE));
-      float kk[EPL], rr[EPL], aa[EPL], zz[EPL];
-      float ss = 0.f;
 #pragma unroll
-      for (int e = 0; e < EPL; ++e) {
-        const int d = lane + WAVE * e;
-        const bool ok = d < D;
-        const int ch = hd * D + (ok ? d : 0);
-        kk[e] = ok ? ldf(row + k_off + ch) : 0.f;
-        rr[e] = ok ? ldf(row + r_off + ch) : 0.f;
-        aa[e] = ok ? sigmoidf_(ldf(row + a_off + ch) + a_b[ch]) : 0.f;
-        zz[e] = ok ? w0[ch] : 0.f;
-        ss += kk[e] * kk[e];
-      }
-      const int r0 = min(rank, WAVE);
-      for (int j = 0; j < r0; ++j) {
-        const float tj = lane_value(tb0, j);
+    for (int s = 0; s < TPW; ++s) {
+      const int tt = pw + PW * s;
+      if (tt < nc) {
+        const float tb0 = tanhf(b0[s]), tb1 = tanhf(b1[s]);   // tanh of the bottleneck, entry j in lane j % 64
+        float zz[EPL];
+        float ss = 0.f;
 #pragma unroll
         for (int e = 0; e < EPL; ++e) {
           const int d = lane + WAVE * e;
-          if (d < D) zz[e] += (w2_in_lds ? s_w2[j * D + d] : w2[(long)(hd * D + d) * rank + j]) * tj;
+          zz[e] = (d < D) ? w0[hd * D + d] : 0.f;
+          ss += kk[s][e] * kk[s][e];
         }
-      }
-      for (int j = WAVE; j < rank; ++j) {
-        const float tj = lane_value(tb1, j - WAVE);
+        const int r0 = min(rank, WAVE);
+        for (int j = 0; j < r0; ++j) {
+          const float tj = lane_value(tb0, j);
+#pragma unroll
+          for (int e = 0; e < EPL; ++e) {
+            const int d = lane + WAVE * e;
+            if (d < D) zz[e] += (w2_in_lds ? s_w2[j * D + d] : w2[(long)(hd * D + d) * rank + j]) * tj;
+          }
+        }
+        for (int j = WAVE; j < rank; ++j) {
+          const float tj = lane_value(tb1, j - WAVE);
+#pragma unroll
+          for (int e = 0; e < EPL; ++e) {
+            const int d = lane + WAVE * e;
+            if (d < D) zz[e] += (w2_in_lds ? s_w2[j * D + d] : w2[(long)(hd * D + d) * rank + j]) * tj;
+          }
+        }
+        const float inv = 1.f / sqrtf(wave_reduce_sum(ss) + 1e-6f);
 #pragma unroll
         for (int e = 0; e < EPL; ++e) {
           const int d = lane + WAVE * e;
-          if (d < D) zz[e] += (w2_in_lds ? s_w2[j * D + d] : w2[(long)(hd * D + d) * rank + j]) * tj;
+          const bool ok = d < D;
+          const float u = kk[s][e] * inv;
+          const float a = ok ? sigmoidf_(ar[s][e] + a_b[hd * D + d]) : 0.f;
+          s_r[b][tt][d] = rr[s][e];
+          s_k[b][tt][d] = kk[s][e];
+          s_u[b][tt][d] = u;
+          s_au[b][tt][d] = a * u;
+          s_w[b][tt][d] = ok ? expf(decay_c * sigmoidf_(zz[e])) : 0.f;
         }
+        if (lane < DR_COLS) s_v[b][tt][lane] = vr[s];
       }
-      const float inv = 1.f / sqrtf(wave_reduce_sum(ss) + 1e-6f);
-#pragma unroll
-      for (int e = 0; e < EPL; ++e) {
-        const int d = lane + WAVE * e;
-        const bool ok = d < D;
-        const float u = kk[e] * inv;
-        s_r[b][tt][d] = rr[e];
-        s_k[b][tt][d] = kk[e];
-        s_u[b][tt][d] = u;
-        s_au[b][tt][d] = aa[e] * u;
-        s_w[b][tt][d] = ok ? expf(decay_c * sigmoidf_(zz[e])) : 0.f;
-      }
-      const int cc = ct * DR_COLS + lane;
-      s_v[b][tt][lane] = (cc < D) ? ldf(row + v_off + hd * D + cc) : 0.f;
     }
   };
 
   // ---- consumer state ----
-  const int c = (wave & 3) * 16 + (lane & 15), rg = lane >> 4;
+  const int rg = lane & 15, c = (wave & 3) * 4 + (lane >> 4);
   const int col = ct * DR_COLS + c;
   const bool colok = col < D;
   const long slot = slots[r];
@@ -132,13 +157,18 @@ __global__ __launch_bounds__(DR_NT) void delta_rule_kernel(
       S[i] = (row < D && colok) ? sp[(long)row * D + col] : 0.f;
     }
   } else if (nchunks > 0) {
-    stage(0, 0);
+    load(0);
+    finish(0, 0);
+    if (nchunks > 1) load(1);
   }
   __syncthreads();
   for (int ci = 0; ci < nchunks; ++ci) {
     const int b = ci & 1;
     if (producer) {
-      if (ci + 1 < nchunks) stage(ci + 1, b ^ 1);
+      if (ci + 1 < nchunks) {
+        finish(ci + 1, b ^ 1);
+        if (ci + 2 < nchunks) load(ci + 2);
+      }
     } else {
       const int tc = t0 + ci * CH;
       const int nc = min(CH, t1 - tc);
@@ -146,26 +176,26 @@ __global__ __launch_bounds__(DR_NT) void delta_rule_kernel(
       for (int tt = 0; tt < nc; ++tt) {
         const float vv = s_v[b][tt][c];
         const float* pu = &s_u[b][tt][rg * RPT];
-        const float* pw = &s_w[b][tt][rg * RPT];
+        const float* pw_ = &s_w[b][tt][rg * RPT];
         const float* pa = &s_au[b][tt][rg * RPT];
         const float* pk = &s_k[b][tt][rg * RPT];
         const float* pr = &s_r[b][tt][rg * RPT];
-        float d0 = 0.f, d1 = 0.f, d2 = 0.f, d3 = 0.f;
+        float d0 = 0.f, d1 = 0.f;
 #pragma unroll
-        for (int i = 0; i < RPT; i += 4) {
-          d0 += pu[i] * S[i]; d1 += pu[i + 1] * S[i + 1]; d2 += pu[i + 2] * S[i + 2]; d3 += pu[i + 3] * S[i + 3];
+        for (int i = 0; i < RPT; i += 2) {
+          d0 += pu[i] * S[i];
+          d1 += pu[i + 1] * S[i + 1];
         }
-        const float dot = sum_row_groups((d0 + d1) + (d2 + d3));
-        float p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;
+        const float dot = sum_row(d0 + d1);
+        float p0 = 0.f, p1 = 0.f;
 #pragma unroll
-        for (int i = 0; i < RPT; i += 4) {
-          S[i] = pw[i] * S[i] - pa[i] * dot + pk[i] * vv;
-          S[i + 1] = pw[i + 1] * S[i + 1] - pa[i + 1] * dot + pk[i + 1] * vv;
-          S[i + 2] = pw[i + 2] * S[i + 2] - pa[i + 2] * dot + pk[i + 2] * vv;
-          S[i + 3] = pw[i + 3] * S[i + 3] - pa[i + 3] * dot + pk[i + 3] * vv;
-          p0 += pr[i] * S[i]; p1 += pr[i + 1] * S[i + 1]; p2 += pr[i + 2] * S[i + 2]; p3 += pr[i + 3] * S[i + 3];
+        for (int i = 0; i < RPT; i += 2) {
+          S[i] = pw_[i] * S[i] - pa[i] * dot + pk[i] * vv;
+          S[i + 1] = pw_[i + 1] * S[i + 1] - pa[i + 1] * dot + pk[i + 1] * vv;
+          p0 += pr[i] * S[i];
+          p1 += pr[i + 1] * S[i + 1];
         }
-        const float part = sum_row_groups((p0 + p1) + (p2 + p3));
+        const float part = sum_row(p0 + p1);
         if (rg == 0 && colok) o[((long)(tc + tt) * H + hd) * D + col] = part;
       }
     }
@@ -224,16 +254,16 @@ void delta_rule_scan(torch::Tensor proj, int64_t r_off, int64_t k_off, int64_t v
   const size_t w2_bytes = (size_t)D * rank * sizeof(float);
   const int w2_in_lds = w2_bytes <= 16 * 1024;
   const size_t smem = w2_in_lds ? w2_bytes : 0;
-#define DR_LAUNCH(DMAX, CH)                                                                                    \
-  hipLaunchKernelGGL((delta_rule_kernel<T, DMAX, CH>), grid, dim3(DR_NT), smem, stream,                        \
+#define DR_LAUNCH(DMAX, CH, PW)                                                                                \
+  hipLaunchKernelGGL((delta_rule_kernel<T, DMAX, CH, PW>), grid, dim3(DR_CONS + PW * WAVE), smem, stream,      \
       (const T*)proj.data_ptr(), (long)proj.stride(0), (int)r_off, (int)k_off, (int)v_off, (int)a_off,         \
       (int)w_off, (int)rank, w2.data_ptr<float>(), w0.data_ptr<float>(), a_b.data_ptr<float>(),                \
       state.data_ptr<float>(), cu.data_ptr<int>(), slots.data_ptr<int>(), o.data_ptr<float>(), (int)H, (int)D, \
       w2_in_lds)
   RAGGED_DISPATCH(proj, {
-    if (D <= 64) DR_LAUNCH(64, 8);
-    else if (D <= 128) DR_LAUNCH(128, 8);
-    else DR_LAUNCH(256, 4);
+    if (D <= 64) DR_LAUNCH(64, 8, 8);
+    else if (D <= 128) DR_LAUNCH(128, 8, 8);
+    else DR_LAUNCH(256, 4, 4);
     const int TH = T_ * H;
     hipLaunchKernelGGL((delta_out_kernel<T>), dim3((TH + 3) / 4), dim3(256), 0, stream, o.data_ptr<float>(),
         (const T*)proj.data_ptr(), (long)proj.stride(0), (int)g_off, norm_w.data_ptr<float>(), (float)eps,
