@@ -104,7 +104,7 @@ torch::Tensor expert_pairs(torch::Tensor h, torch::Tensor ids, torch::Tensor wgu
   const int K = ids.size(1);
   TORCH_CHECK(wgu.size(1) == 2 * F && wgu.size(2) == W && wd.size(0) == E && wd.size(1) == W && wd.size(2) == F);
   TORCH_CHECK(W % 8 == 0 && F % 8 == 0, "pair kernels take widths that are multiples of 8");
-  TORCH_CHECK((size_t)std::max(W, F) * sizeof(float) <= 64 * 1024, "input vector above the LDS staging size");
+  TORCH_CHECK((size_t)std::max(W, F) * sizeof(float) <= 60 * 1024, "input vector above the LDS staging size");
   const int N = T_ * K;
   auto out = torch::empty({N, W}, h.options());
   if (N == 0) return out;

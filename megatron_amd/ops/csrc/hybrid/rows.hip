@@ -87,7 +87,7 @@ std::vector<torch::Tensor> residual_group_norm(torch::Tensor x, torch::Tensor y,
   if (T_ == 0) return {ha, hb};
   auto stream = at::cuda::getCurrentHIPStream();
   const size_t smem = (size_t)W * sizeof(float);
-  TORCH_CHECK(smem <= 96 * 1024, "row too wide for the norm kernel");
+  TORCH_CHECK(smem <= 60 * 1024, "row too wide for the norm kernel");
 #define GN_LAUNCH(TY, TO)                                                                                        \
   hipLaunchKernelGGL((residual_group_norm_kernel<TY, TO>), dim3(T_), dim3(256), smem, stream, x.data_ptr<float>(), \
       has_y ? (const TY*)y.data_ptr() : (const TY*)nullptr, wa.data_ptr<float>(),                                \
@@ -269,7 +269,7 @@ std::vector<torch::Tensor> moe_router(torch::Tensor h, torch::Tensor wr, int64_t
   TORCH_CHECK(top >= 1 && top <= RT_MAX_TOP && top <= E, "experts chosen per token");
   TORCH_CHECK(groups >= 1 && groups <= RT_MAX_GROUPS && E % groups == 0 && keep >= 1 && keep <= groups);
   TORCH_CHECK(groups == 1 || keep * (E / groups) >= top, "the kept groups hold fewer experts than are chosen");
-  TORCH_CHECK((size_t)W * sizeof(float) <= 64 * 1024, "row too wide for the router kernel");
+  TORCH_CHECK((size_t)W * sizeof(float) <= 60 * 1024, "row too wide for the router kernel");
   auto ids = torch::empty({T_, top}, h.options().dtype(at::kInt));
   auto wts = torch::empty({T_, top}, h.options().dtype(at::kFloat));
   auto extra = torch::empty({T_, rows - E}, h.options().dtype(at::kFloat));

@@ -320,7 +320,7 @@ def expert_pairs_ok(h, top, ff) -> bool:
     """Steps with few pairs (decoding) skip the sort by expert: see csrc/hybrid/experts.hip."""
     return (h.is_cuda and _H is not None and os.environ.get("MEGATRON_AMD_FORCE_REFERENCE", "0") != "1"
             and h.shape[0] * top <= PAIR_PATH_MAX and h.shape[1] % 8 == 0 and ff % 8 == 0
-            and max(h.shape[1], ff) <= 16384)
+            and max(h.shape[1], ff) <= 15360)
 
 
 def expert_pairs(h, ids, w_gate_up, w_down, limit, alpha):
@@ -331,6 +331,6 @@ def expert_pairs(h, ids, w_gate_up, w_down, limit, alpha):
 
 def moe_router(h, w_router, experts, top, groups, keep, scale):
     """-> (ids [T, top] int32, weights [T, top] fp32, raw logits of the rows beyond the experts)"""
-    if _native_h(h) and h.shape[1] <= 16384 and w_router.shape[0] <= 512:
+    if _native_h(h) and h.shape[1] <= 15360 and w_router.shape[0] <= 512:
         return _H.moe_router(h, w_router, int(experts), int(top), int(groups), int(keep), float(scale))
     return ref.moe_router(h, w_router, experts, top, groups, keep, scale)

@@ -50,7 +50,7 @@ def test_embed_and_group_norm(dtype, groups):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("shape", [(4, 2, 24, 24, 9, 4), (3, 3, 80, 80, 5, 1), (6, 1, 136, 136, 64, 7), (2, 2, 16, 16, 1, 3),
-                                   (8, 2, 64, 64, 40, 6)])
+                                   (8, 2, 64, 64, 40, 6), (2, 1, 12, 12, 5, 2)])
 @pytest.mark.parametrize("starts", [STARTS, [0, 300, 130, 3, 517]], ids=["short", "long"])
 def test_pooled_window_attention(dtype, shape, starts):
     """heads, kv heads, dim, vdim, window, pool; page 16: pooled rows and windows cross pages;

@@ -28,12 +28,12 @@ def serve_model_dir(args):
 
     device = torch.device("cuda") if torch.cuda.is_available() else torch.device("cpu")
     dtype = torch.bfloat16 if args.serve_dtype == "bfloat16" else torch.float32
+    model = build_from_dir(args.model_dir, dtype=dtype, device=device)
     if device.type == "cuda":
         from megatron_amd.ops import ragged
 
-        if ragged._C is None:
-            ragged.build_ragged_ops()
-    model = build_from_dir(args.model_dir, dtype=dtype, device=device)
+        # only the kernel extensions this model's layers use are compiled on first use
+        ragged.ensure_built(getattr(model, "native_extensions", ("ragged",)))
     tokenizer = (build_tokenizer(args.tokenizer_type, args.tokenizer_model, model.config.vocab_size)
                  if args.tokenizer_model else None)
     engine = DynamicInferenceEngine(model, tokenizer, num_blocks=args.kv_blocks,
