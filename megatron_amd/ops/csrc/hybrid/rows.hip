@@ -313,12 +313,53 @@ torch::Tensor clamped_glu(torch::Tensor gu, double limit, double alpha) {
 // y[t] = sum_k w[t,k] down[inv[t,k]] + sigmoid(gate[t]) shared[t] + add[t]   (fp32)
 // ---------------------------------------------------------------------------
 template <typename T>
+__device__ __forceinline__ void load8_(const T* p, float* v);
+template <>
+__device__ __forceinline__ void load8_<bf16>(const bf16* p, float* v) {
+  const short8 x = *reinterpret_cast<const short8*>(p);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = sbf2f(x[i]);
+}
+template <>
+__device__ __forceinline__ void load8_<float>(const float* p, float* v) {
+  const float4v a = *reinterpret_cast<const float4v*>(p), b = *reinterpret_cast<const float4v*>(p + 4);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { v[i] = a[i]; v[4 + i] = b[i]; }
+}
+
+// VEC: 8 elements per thread and pass with 16/32-byte accesses (W a multiple of 8), else one
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void moe_combine_kernel(
     const T* __restrict__ down, const int* __restrict__ inv, const float* __restrict__ wts,
     const T* __restrict__ shared, const float* __restrict__ gate, const T* __restrict__ add,
     float* __restrict__ y, int W, int K) {
   const long t = blockIdx.x;
   const float sg = shared != nullptr ? sigmoidf_(gate[t]) : 0.f;
+  if (VEC) {
+    for (int c = threadIdx.x * 8; c < W; c += 256 * 8) {
+      float a[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, v[8];
+      for (int k = 0; k < K; ++k) {
+        const float w = wts[t * K + k];
+        load8_<T>(down + (long)inv[t * K + k] * W + c, v);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) a[i] += w * v[i];
+      }
+      if (shared != nullptr) {
+        load8_<T>(shared + t * W + c, v);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) a[i] += sg * v[i];
+      }
+      if (add != nullptr) {
+        load8_<T>(add + t * W + c, v);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) a[i] += v[i];
+      }
+      float4v* yp = reinterpret_cast<float4v*>(y + t * W + c);
+      yp[0] = float4v{a[0], a[1], a[2], a[3]};
+      yp[1] = float4v{a[4], a[5], a[6], a[7]};
+    }
+    return;
+  }
   for (int c = threadIdx.x; c < W; c += 256) {
     float a = 0.f;
     for (int k = 0; k < K; ++k) a += wts[t * K + k] * ldf(down + (long)inv[t * K + k] * W + c);
@@ -346,9 +387,15 @@ torch::Tensor moe_combine(torch::Tensor down, torch::Tensor inv, torch::Tensor w
   auto y = torch::empty({T_, W}, down.options().dtype(at::kFloat));
   if (T_ == 0) return y;
   auto stream = at::cuda::getCurrentHIPStream();
-  RAGGED_DISPATCH(down, hipLaunchKernelGGL((moe_combine_kernel<T>), dim3(T_), dim3(256), 0, stream,
-      (const T*)down.data_ptr(), inv.data_ptr<int>(), wts.data_ptr<float>(),
-      has_s ? (const T*)shared.data_ptr() : (const T*)nullptr, has_s ? gate.data_ptr<float>() : (const float*)nullptr,
-      has_a ? (const T*)add.data_ptr() : (const T*)nullptr, y.data_ptr<float>(), W, K));
+#define MC_LAUNCH(VEC)                                                                                          \
+  hipLaunchKernelGGL((moe_combine_kernel<T, VEC>), dim3(T_), dim3(256), 0, stream, (const T*)down.data_ptr(),    \
+      inv.data_ptr<int>(), wts.data_ptr<float>(), has_s ? (const T*)shared.data_ptr() : (const T*)nullptr,       \
+      has_s ? gate.data_ptr<float>() : (const float*)nullptr, has_a ? (const T*)add.data_ptr() : (const T*)nullptr, \
+      y.data_ptr<float>(), W, K)
+  RAGGED_DISPATCH(down, {
+    if (W % 8 == 0) MC_LAUNCH(true);
+    else MC_LAUNCH(false);
+  });
+#undef MC_LAUNCH
   return y;
 }

@@ -132,11 +132,12 @@ def test_moe_route(cfg):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_glu_and_combine(dtype):
+@pytest.mark.parametrize("W", [40, 36])
+def test_glu_and_combine(dtype, W):
     R = _need()
 
     def run(dev, dt):
-        T, K, W, F_ = 9, 3, 40, 24
+        T, K, F_ = 9, 3, 24
         gu = _rand((T * K, 2 * F_), dt, dev, 2.0)
         y = R.clamped_glu(gu, 1.5, 1.702, dt)
         down = _rand((T * K, W), dt, dev)
