@@ -12,9 +12,10 @@ Optional shared expert of the same form for every token, times
 sigmoid(w_sg . h); its gate row rides in the fp32 router GEMM.
 
 Step: one router kernel (fp32 logits of [router; shared gate], scores, selection), then
-  * many pairs (prompt portions): the (token, choice) pairs are sorted by expert
-    and each expert with work runs its gate/up and down products on its slice
-    (vendor GEMMs; the pair counts are the step's one host read),
+  * many pairs (prompt portions): the (token, choice) pairs are sorted by expert;
+    bf16 runs one grouped GEMM per linear over the sorted pairs with the group
+    ends on the device (no host read); fp32 and unaligned sizes run each expert
+    with work on its slice (vendor GEMMs; the pair counts are one host read),
   * few pairs (decoding): two kernels in which every pair streams its expert's
     matrices (ops.ragged.expert_pairs), no sort and no host read,
 and one kernel forms sum_k weight_k down_k + sigmoid(gate) shared + add in fp32.
@@ -22,6 +23,7 @@ and one kernel forms sum_k weight_k down_k + sigmoid(gate) shared + add in fp32.
 
 from __future__ import annotations
 
+import os
 from typing import Optional
 
 import torch
@@ -55,6 +57,13 @@ class RoutedExpertsMLP(nn.Module):
         """-> (ids [T, top], weights [T, top], the shared expert's gate logit [T, 1] or [T, 0])"""
         return R.moe_router(h, self.w_router, self.experts, self.top, self.groups, self.keep, self.route_scale)
 
+    def _grouped_ok(self, h: torch.Tensor) -> bool:
+        """bf16 on the GPU with 16-byte aligned rows: the grouped GEMM the training-side
+        expert layer uses (ops.grouped_linear), here with its offsets left on the device."""
+        return (h.is_cuda and h.dtype == torch.bfloat16 and hasattr(torch, "_grouped_mm")
+                and h.shape[1] % 8 == 0 and self.ff % 8 == 0
+                and os.environ.get("MEGATRON_AMD_NO_TORCH_GROUPED", "0") != "1")
+
     def forward(self, h: torch.Tensor, add: Optional[torch.Tensor] = None) -> torch.Tensor:
         """h [T, hidden] in the compute dtype -> fp32 [T, hidden] (+ add)."""
         T, K, E = h.shape[0], self.top, self.experts
@@ -73,13 +82,20 @@ class RoutedExpertsMLP(nn.Module):
         order = torch.argsort(flat, stable=True)              # pairs sorted by expert
         inv = torch.empty_like(order)
         inv[order] = torch.arange(order.numel(), device=order.device)
-        counts = torch.bincount(flat, minlength=E).tolist()   # the step's host read
         xs = h.index_select(0, torch.div(order, K, rounding_mode="floor"))
-        down = torch.empty(T * K, h.shape[1], dtype=h.dtype, device=h.device)
-        at = 0
-        for e, n in enumerate(counts):
-            if n:
-                gu = F.linear(xs[at:at + n], self.w_gate_up[e])
-                down[at:at + n] = F.linear(R.clamped_glu(gu, self.limit, self.alpha, h.dtype), self.w_down[e])
-                at += n
+        if self._grouped_ok(h):
+            # one grouped GEMM per linear over the sorted pairs, group ends on the device: no host read
+            offs = torch.cumsum(torch.bincount(flat, minlength=E), 0).to(torch.int32)
+            gu = torch._grouped_mm(xs, self.w_gate_up.transpose(1, 2), offs=offs)
+            down = torch._grouped_mm(R.clamped_glu(gu, self.limit, self.alpha, h.dtype),
+                                     self.w_down.transpose(1, 2), offs=offs)
+        else:
+            counts = torch.bincount(flat, minlength=E).tolist()   # the step's host read
+            down = torch.empty(T * K, h.shape[1], dtype=h.dtype, device=h.device)
+            at = 0
+            for e, n in enumerate(counts):
+                if n:
+                    gu = F.linear(xs[at:at + n], self.w_gate_up[e])
+                    down[at:at + n] = F.linear(R.clamped_glu(gu, self.limit, self.alpha, h.dtype), self.w_down[e])
+                    at += n
         return R.moe_combine(down, inv.view(T, K).to(torch.int32), weights, shared, gate, add)
