@@ -19,7 +19,7 @@ constexpr int DR_MAX_RANK = 128;     // decay bottleneck
 constexpr int DP_TOK = 16;           // tokens per workgroup of the prep kernel (4 per wave)
 
 // x summed over the 16 lanes of its wave row, in every lane: four rotations inside
-// the row (DPP modifiers of the adds: VALU only, no LDS round trip)
+// the row (DPP modifiers of the adds: VALU only, nothing passes through LDS)
 __device__ __forceinline__ float sum_row(float x) {
   x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x128, 0xf, 0xf, false));   // row_ror:8
   x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x124, 0xf, 0xf, false));   // row_ror:4

@@ -247,7 +247,7 @@ def test_delta_rule_removes_along_the_key():
     assert_close(S.T @ k, (k @ k) * v2, 1e-4)
 
 
-@pytest.mark.parametrize("E,top,groups,keep", [(6, 2, 3, 2), (8, 1, 1, 1), (12, 4, 4, 3), (6, 3, 6, 4), (9, 3, 3, 3)])
+@pytest.mark.parametrize("E,top,groups,keep", [(6, 2, 3, 2), (8, 1, 1, 1), (15, 4, 5, 3), (6, 3, 6, 4), (9, 3, 3, 3)])
 def test_router_alone(E, top, groups, keep):
     from megatron_amd.ops import ragged as R
 
@@ -574,7 +574,7 @@ def test_gpu_grouped_and_looped_expert_paths_agree():
 
     torch.manual_seed(0)
     W, E, F_ = 64, 12, 40
-    mlp = RoutedExpertsMLP(W, E, 2, F_, 1.5, groups=4, keep=1, route_scale=1.5, shared_ff=24, shared_limit=1.0)
+    mlp = RoutedExpertsMLP(W, E, 2, F_, 1.25, groups=4, keep=1, route_scale=1.75, shared_ff=24, shared_limit=0.75)
     with torch.no_grad():
         for p in mlp.parameters():
             p.copy_(torch.randn(p.shape) * 0.2)
