@@ -130,9 +130,25 @@ __global__ __launch_bounds__(256) void pooled_window_attn_mfma_kernel(
   // Register-staged tile pipeline: the global loads of tile t+1 are issued right
   // after tile t became visible in LDS and are waited for when they are written
   // to LDS at the top of the next iteration.
+  // pages that are a multiple of the key tile hold a token tile in one piece: one scalar
+  // page lookup per tile instead of two divisions per staged row
+  const bool whole = (bs % PW_KT) == 0;
+  long s_off[NSTG];                               // offset inside a tile whose rows are consecutive
+#pragma unroll
+  for (int k = 0; k < NSTG; ++k) s_off[k] = (long)s_row[k] * width + s_col[k];
   auto issue = [&](int tile) {
     const bool is_pooled = tile < npt;
     const int base = is_pooled ? tile * PW_KT : (jt0 + tile - npt) * PW_KT;
+    if (!is_pooled && whole) {
+      const bf16* rows = pool + ((long)tab[base / bs] * bs + (base % bs)) * width;
+#pragma unroll
+      for (int k = 0; k < NSTG; ++k) {
+        short8 v = short8{0, 0, 0, 0, 0, 0, 0, 0};
+        if (s_col[k] >= 0 && base + s_row[k] <= p_max) v = *reinterpret_cast<const short8*>(rows + s_off[k]);
+        stg[k] = v;
+      }
+      return;
+    }
 #pragma unroll
     for (int k = 0; k < NSTG; ++k) {
       short8 v = short8{0, 0, 0, 0, 0, 0, 0, 0};

@@ -1,10 +1,16 @@
-"""Ragged-batch sequence ops: embedding with hashed bigrams, hyper-connection
-stream mixing fused with RMS norm, residual causal convolution with carried
-taps, minGRU and mLSTM recurrences with per-request state slots, latent-cache
-attention with a softmax sink, xIELU.
+"""Ragged-batch sequence ops.
+
+``_ragged_ops``: embedding with hashed bigrams, hyper-connection stream mixing
+fused with RMS norm, residual causal convolution with carried taps, minGRU and
+mLSTM recurrences with per-request state slots, latent-cache attention with a
+softmax sink, xIELU.
+``_hybrid_ops``: embedding into a plain fp32 residual, residual add fused with
+grouped RMS norm, whole-projection q/k norm with cache store, pooled-block
+completion and attention over a sliding window plus pooled blocks, generalized
+delta rule, expert routing, clamped GLU, pair-streaming experts, expert combine.
 
 Dispatch rule (same as megatron_amd.ops): tensors on a HIP device run the
-CDNA4 kernels of the ``_ragged_ops`` extension (csrc/ragged/*.hip) and RAISE
+CDNA4 kernels of the extension (csrc/ragged/*.hip, csrc/hybrid/*.hip) and RAISE
 when it is not built; CPU tensors run the torch implementations in
 ``ragged_reference`` so every path tests without a GPU.
 MEGATRON_AMD_FORCE_REFERENCE=1 forces the torch path (numerics tests).
