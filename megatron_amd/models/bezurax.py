@@ -58,8 +58,13 @@ class BezuraxConfig:
 
     def owner(self, i: int) -> int:
         """the layer whose weights layer i uses"""
-        src = self.layers[i].get("weights_of")
-        return i if src is None else int(src)
+        seen = set()
+        while self.layers[i].get("weights_of") is not None:
+            if i in seen:
+                raise ValueError(f"layers share weights in a circle at layer {i}")
+            seen.add(i)
+            i = int(self.layers[i]["weights_of"])
+        return i
 
 
 class BezuraxBlock(nn.Module):
