@@ -409,14 +409,17 @@ def test_one_key_inside_or_outside_changes_the_answer():
     assert (a - c).abs().max() > 50 * 2e-4 * a.abs().max()
 
 
-def test_far_key_is_seen_through_its_block():
+@pytest.mark.parametrize("P,first", [(4, 40), (3, 63), (5, 20)])      # blocks inside a page (8), across a page border
+@pytest.mark.parametrize("decode", [False, True])
+def test_far_key_is_seen_through_its_block(P, first, decode):
     """A key hundreds of tokens back that wins the softmax: its block's mean
     carries it.  The attention op on a designed cache: every key is small
-    except one far block's, which is aligned with the query."""
+    except one far block's, which is aligned with the last query; the query is
+    part of the prompt, or decoded alone after it."""
     from megatron_amd.ops import ragged as R
 
     H = G = 1
-    D, window, P, page, n = 8, 16, 4, 8, 300
+    D, window, page, n = 8, 16, 8, 300
     rpp = (page + P - 1) // P
     ctx = HybridInferenceContext({"c": 2 * D, "c.pooled": (2 * D, rpp)}, {}, 40, page, 1, dtype=torch.float32, device="cpu")
     table = ctx.allocator.allocate((n + page - 1) // page)[::-1]
@@ -424,19 +427,21 @@ def test_far_key_is_seen_through_its_block():
     proj = torch.randn(n, 2 * D) * 0.05                             # [q | k], v = k
     direction = torch.zeros(D)
     direction[3] = 1.0
-    far = 41                                                        # block 10 = positions 40..43
-    proj[40:44, D:] += 3.0 * direction
+    assert first % P == 0 and first + P <= n - window
+    proj[first:first + P, D:] += 3.0 * direction                    # one whole block
     proj[n - 1, :D] = 5.0 * direction
-    ctx.begin_batch([n], [0], [0], [table])
     ones = torch.ones(D)
-    q = R.qk_norm_store(proj, 0, D, D, D, D, D, ones, ones, 1e-6, ctx.pools["c"], ctx.batch)
-    R.pool_blocks(ctx.pools["c"], ctx.pools["c.pooled"], P, rpp, ctx.batch)
     out = torch.zeros(n, D)
-    R.pooled_window_attention(q, ctx.pools["c"], ctx.pools["c.pooled"], H, G, D, D, 4.0, window, P, rpp,
-                              ctx.batch, out, 0, 1.0)
-    want_v = proj[40:44, D:].mean(0)
+    for a, b in ([(0, n - 1), (n - 1, n)] if decode else [(0, n)]):
+        ctx.begin_batch([b - a], [a], [0], [table])
+        q = R.qk_norm_store(proj[a:b], 0, D, D, D, D, D, ones, ones, 1e-6, ctx.pools["c"], ctx.batch)
+        R.pool_blocks(ctx.pools["c"], ctx.pools["c.pooled"], P, rpp, ctx.batch)
+        R.pooled_window_attention(q, ctx.pools["c"], ctx.pools["c.pooled"], H, G, D, D, 4.0, window, P, rpp,
+                                  ctx.batch, out[a:b], 0, 1.0)
+    want_v = proj[first:first + P, D:].mean(0)
     assert_close(out[n - 1], want_v, 2e-2)                          # the far block dominates the answer
-    assert far < n - window
+    # and the same query with the block's keys left small answers something else
+    assert (out[n - 2] - want_v).abs().max() > 0.5
 
 
 def test_first_tokens():
